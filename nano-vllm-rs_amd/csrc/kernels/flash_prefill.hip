@@ -43,6 +43,7 @@ struct FlashParams {
     float *part_o, *part_ml;
     const int32_t *srows, *scount;     // optional: only the rows srows[0 .. *scount) of the batch share the prefix (row srows[0] names its blocks)
     const float *r1, *r2, *sink; int64_t ldo;   // PEN instantiations: distance penalty and sink per head (FlashArgs); ldo: output row stride in elements
+    int32_t window;                              // PEN instantiations: > 0, a query sees only the keys less than `window` positions back
 };
 
 
@@ -145,7 +146,8 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, g4 = lane >> 4;
     // SHARED: blockIdx.y cuts the shared keys into partitions of shared_len tokens (more workgroups than 8 per kv head at 512 sequences)
-    const int kv_start = SHARED ? (int)blockIdx.y * p.shared_len : 0;
+    // (a window: the first step is the one that holds the first key the tile's first query sees)
+    const int kv_start = SHARED ? (int)blockIdx.y * p.shared_len : ((PEN && p.window > 0) ? max(tile.pos0 - p.window + 1, 0) / KT * KT : 0);
     const int kv_end = SHARED ? kv_start + p.shared_len : tile.pos0 + tile.nq;
 
     // the wave's two query tiles: head and position block
@@ -266,10 +268,11 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
     // PEN: the scores are moved to the base-2 domain before the softmax (s <- s c2 - r1 log2(1 + r2 (i - j)): r1 ln(x) log2(e) = r1 log2(x), one v_log_f32 per
     // score), so the factor of the exponent is 1 from there on; the sink is the running maximum's first value and a 1 in the running sum
     const float cs = PEN ? 1.0f : c2;
+    const bool lin = PEN && p.r1 && !p.r2;                       // r1 alone: a penalty linear in the distance, r1 (i - j)
     float pr1[NQT], pr2[NQT];
 #pragma unroll
     for (int t = 0; t < NQT; ++t) {
-        pr1[t] = (PEN && p.r1) ? p.r1[head[t]] : 0.f; pr2[t] = (PEN && p.r2) ? p.r2[head[t]] : 0.f;
+        pr1[t] = (PEN && p.r1) ? p.r1[head[t]] * (lin ? 1.44269504088896340736f : 1.0f) : 0.f; pr2[t] = (PEN && p.r2) ? p.r2[head[t]] : 0.f;
         if (PEN && p.sink) { m[t] = p.sink[head[t]] * 1.44269504088896340736f; ol[t] = (float4_t){1.f, 1.f, 1.f, 1.f}; }
     }
     half8_t ones;
@@ -319,8 +322,10 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
                 for (int mt = 0; mt < NMT; ++mt)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float dist = (float)max(qpos[t] - (kt + mt * 16 + g4 * 4 + e), 0);
-                        s[t][mt][e] = fmaf(s[t][mt][e], c2, -pr1[t] * __builtin_amdgcn_logf(fmaf(pr2[t], dist, 1.0f)));
+                        const int di = max(qpos[t] - (kt + mt * 16 + g4 * 4 + e), 0);
+                        const float dist = (float)di;
+                        const float v = fmaf(s[t][mt][e], c2, lin ? -pr1[t] * dist : -pr1[t] * __builtin_amdgcn_logf(fmaf(pr2[t], dist, 1.0f)));
+                        s[t][mt][e] = (p.window > 0 && di >= p.window) ? -INFINITY : v;
                     }
         }
         // causal mask only on steps that reach past the tile's first query (keys kt + mt*16 + g4*4 + e)
@@ -450,8 +455,9 @@ int flash_prefill(const FlashArgs &a, bool paged, hipStream_t s) {
     p.block_tables = a.block_tables; p.max_blocks = a.max_blocks; p.block_size = a.block_size;
     p.bs_shift = (a.block_size > 0 && (a.block_size & (a.block_size - 1)) == 0) ? __builtin_ctz(a.block_size) : -1;
     p.tiles = a.tiles; p.H = a.H; p.KVH = a.KVH; p.scale = a.scale; p.out = (half_t *)a.out;
-    p.r1 = a.r1; p.r2 = a.r2; p.sink = a.sink; p.ldo = a.ldo ? a.ldo : (int64_t)a.H * a.D;
-    const bool pen = (a.r1 && a.r2) || a.sink;
+    p.r1 = a.r1; p.r2 = a.r2; p.sink = a.sink; p.ldo = a.ldo ? a.ldo : (int64_t)a.H * a.D; p.window = a.window;
+    const bool pen = a.r1 || a.sink;
+    if (a.window > 0 && !a.sink) return nvr::fail(NVR_ERR_UNSUPPORTED, "flash_prefill: a window needs the sink form (a step may hold no visible key)");
     if (pen && !paged) return nvr::fail(NVR_ERR_UNSUPPORTED, "flash_prefill: the penalty / sink form reads K and V through block tables");
     const int G = a.H / a.KVH;
     dim3 grid((unsigned)((int64_t)a.ntiles * a.KVH)), block(64 * FLASH_WAVES);

@@ -61,7 +61,9 @@ struct FlashArgs {
     // Optional (all zero: plain softmax attention).  A distance penalty and a sink per head: score = q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)), and the
     // softmax denominator also holds exp(sink[h]) (a term with no key and no value).  r1 / r2 together, sink on its own, each [H] f32 on the device.
     // ldo: elements between the output rows of consecutive query rows (0: H * D)
+    // r1 without r2: a penalty linear in the distance, r1[h] * (i - j).  window > 0 (with a sink): a query sees only the keys less than `window` positions back.
     const float *r1, *r2, *sink; int64_t ldo;
+    int32_t window;
 };
 
 // Config.dtype = "float32": attention arguments of the f32 path (kernels/f32_path.hip)

@@ -50,6 +50,9 @@ struct SinkAttnArgs {
     int32_t v_grouped;                       // tiled form: value pages in groups of 8 keys per column (kv_store's v_grouped), else row-major [.][G][Dv]
     int64_t vld;                             // general form: elements between the value rows of consecutive key/value heads (0: Dv); with vc = kc and vld = D the values
                                              // are the first Dv numbers of the key rows (one cached row per token serves as key and value)
+    const float *slope;                      // a linear distance penalty instead of the logarithmic one: score -= slope[h] * (i - j) (null: none; not together with r1 / r2).
+                                             // The tiled form takes it as its table (linear_penalty_table)
+    int32_t window;                          // > 0: position i sees only the keys j with i - j < window (itself and the window - 1 before it); 0: every key j <= i
 };
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);     // any shape; a context that fits the LDS score buffer
 // The same on the matrix cores (bf16 operands, D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16).  tiles (device, built by the host): tile i covers the
@@ -59,6 +62,8 @@ struct AttnTile { int32_t seq, row0; };
 bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16, int block_size);   // (pages of a multiple of 8 tokens)
 // tab[h][d] = r1[h] * ln(1 + r2[h] * d) * log2(e) for d < n: the penalty the tiled form subtracts in the base-2 domain
 int penalty_table(const float *r1, const float *r2, int64_t H, int64_t n, float *tab, hipStream_t s);
+// tab[h][d] = slope[h] * d * log2(e): the same table for a linear penalty
+int linear_penalty_table(const float *slope, int64_t H, int64_t n, float *tab, hipStream_t s);
 size_t sink_attention_workspace_bytes(int max_workgroups);
 int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, int nsplit, void *workspace, size_t workspace_bytes, hipStream_t s);
 
@@ -73,6 +78,10 @@ struct RetentionArgs {
     // gated form (az not null): the decay of token t and key channel d of head h is sigmoid(az[t][h * D + d] + abias[h * D + d])^inv_tau, all in f32 from rows of
     // the operand type (stride ldz), instead of decay[h]; q is scaled by qscale
     const void *az; int64_t ldz; const float *abias; float inv_tau, qscale;
+    // token-gated form (tok_gate not null): S <- keep S + take k v^T with the two f32 numbers (keep, take) of token t and head h at tok_gate[(t * H + h) * 2]
+    // (instead of decay[h]); q is scaled by qscale.  v_ones: the last v_ones of the Dv value columns are not read from proj (whose value rows hold Dv - v_ones
+    // numbers per head): their value is 1 for every token, so that the state's column is the gated running sum of the keys and o's column its product with q.
+    const float *tok_gate; int32_t v_ones;
 };
 int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s);
 // out[t][h*Dv + c] = o[t][h][c] / rms(o[t][h][:]) * w[c] * silu(gate[t][h*Dv + c]); gate: rows of the operand type (stride ldg) from column gcol; w (one weight per
@@ -158,5 +167,49 @@ struct LayerTailArgs {
     const float *wnext; int32_t groups; void *out;
 };
 int layer_tail(const LayerTailArgs &a, bool bf16, hipStream_t s);
+
+// ---------------------------------------------------------------------------------------------------------------------------------------------------
+// Blocks of pre-norm layers with a layer scale (layered_gates.hip): learned positions, an exponentially gated matrix memory, a windowed attention with
+// normed queries / keys / values, an elementwise gated recurrence, and the residual joins.
+
+// x[t] = E[ids[t]] * scale + P[position of row t] (f32 residual stream; P: [positions][W] of the operand type, null: none)
+int embed_pos(const void *E, const void *P, bool bf16, const Batch &b, int64_t W, float scale, float *x, hipStream_t s);
+
+// Exponential gates of a matrix memory, per token and head, from the f32 pre-activations zi = pre[t][h], zf = pre[t][H + h] (row stride ldp) and their biases:
+//   i = cap tanh((zi + bi[h]) / cap), f = log_sigmoid(cap tanh((zf + bf[h]) / cap)), m_t = max(f + m_(t-1), i) with m = 0 before a sequence's first token;
+//   tok_gate[(t * H + h) * 2] = (e^(f + m_(t-1) - m_t), e^(i - m_t)) — retention's token-gated form takes these — and floor[t * H + h] = e^(-m_t).
+// mstate: [slots][H] f32, the running maximum after each sequence's last token so far.
+int exp_gates(const float *pre, int64_t ldp, const float *bi, const float *bf, float cap, const Batch &b, int64_t H, float *mstate, float *tok_gate, float *floor_out,
+              hipStream_t s);
+// The matrix memory's read-out: o rows [T][H][Dv + 1] f32 (retention's output with one column of ones: the last number of a head is n . q);
+//   y = o[:Dv] / (max(|n . q|, floor) + 1e-6), y / rms(y) * w[h * Dv + c] * sigmoid(gate[t][h * Dv + c]) -> out rows (operand type, stride ldo)
+int memory_readout(const float *o, const float *floor_in, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, const float *w, void *out,
+                   int64_t ldo, bool bf16, hipStream_t s);
+
+// Queries, keys and values of an attention whose norms span the projections: in row t of proj (operand type, stride ld)
+//   q (H D numbers at qcol) <- q / rms(q) * wq * (1 + coef ln(floor((p + 1) / every) + 1)), in place (p the row's position; every 0: no temperature);
+//   k (G D numbers at kcol) / rms(k) * wk -> the K page row of the position; v (G heads of Dv at vcol), each head / rms(head) -> the V page row.
+// wq / wk null: that projection is stored as it is.  v_unit false: values as they are.  Page layouts as kv_store.
+struct QkvNormArgs {
+    void *proj; int64_t ld, qcol, kcol, vcol; int32_t H, G, D, Dv; float eps;
+    const float *wq, *wk; bool v_unit; float temp_coef; int32_t temp_every;
+    void *kc, *vc; bool v_grouped;
+};
+int qkv_norm_store(const QkvNormArgs &a, const Batch &b, bool bf16, hipStream_t s);
+
+// Elementwise gated recurrence over the rows of a step: z = sigmoid(proj[zcol + c] + bz[c]), u = proj[ucol + c] + bu[c], cand = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),
+// S <- (1 - z) S + z cand, out[t][c] = S * silu(proj[gcol + c]) (operand type, stride ldo).  state: [slots][N] f32, zero before a sequence's first token.
+int gated_unit(const void *proj, int64_t ld, int64_t zcol, int64_t ucol, int64_t gcol, const float *bz, const float *bu, const Batch &b, int64_t N, float *state, void *out, int64_t ldo,
+               bool bf16, hipStream_t s);
+
+// A sublayer's result joins the stream: x[t][c] += ls[c] * r, r = y1 (y2 null) or (y1 / rms(y1) * w1 + y2 / rms(y2) * w2) / 2 (two branches, each normed over the row);
+// with wn also out[t] = x[t] / rms(x[t]) * wn in the operand type (the next sublayer's input).  y rows of the operand type, strides ld1 / ld2; ls may be null (ones).
+struct JoinArgs { float *x; int64_t T, W; float eps; const float *ls; const void *y1; int64_t ld1; const float *w1; const void *y2; int64_t ld2; const float *w2; const float *wn; void *out; int64_t ldo; };
+int residual_join(const JoinArgs &a, bool bf16, hipStream_t s);
+
+// out = max(z, 0)^2 (rows of F numbers, strides ldz / ldo)
+int relu_squared(const void *z, int64_t ldz, int64_t T, int64_t F, void *out, int64_t ldo, bool bf16, hipStream_t s);
+// y[i] *= c (f32, n numbers)
+int scale_f32(float *y, int64_t n, float c, hipStream_t s);
 
 }}  // namespace nvr::kl

@@ -223,32 +223,35 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
     __syncthreads();
     const CT *kc = (const CT *)a.kc; const CT *vc = (const CT *)a.vc;
     const int32_t *bt = b.block_tables + (int64_t)sq * b.max_blocks;
-    const float r1 = a.r1 ? a.r1[h] : 0.f, r2 = a.r2 ? a.r2[h] : 0.f;
+    const float r1 = a.r1 ? a.r1[h] : 0.f, r2 = a.r2 ? a.r2[h] : 0.f, slope = a.slope ? a.slope[h] : 0.f;
+    const int j0 = a.window > 0 ? max(0, ctx - a.window) : 0;      // first visible key; the score buffer holds the keys j0 .. ctx - 1
+    sc -= j0;
     float mx = a.sink ? a.sink[h] : -INFINITY;
-    for (int j = threadIdx.x; j < ctx; j += 256) {
+    for (int j = j0 + threadIdx.x; j < ctx; j += 256) {
         const int64_t row = (int64_t)bt[j / b.block_size] * b.block_size + j % b.block_size;
         const int64_t base = (row * a.G + kvh) * a.D;
         float dot = 0.f;
         for (int d = 0; d < a.D; ++d) dot += qs[d] * ld_f(kc, base + d);
         float s = dot * a.scale;
         if (a.r1) s -= r1 * log1pf(r2 * (float)(i - j));
+        if (a.slope) s -= slope * (float)(i - j);
         sc[j] = s;
         mx = fmaxf(mx, s);
     }
     mx = block_max<256>(mx, red);
     float sum = 0.f;
-    for (int j = threadIdx.x; j < ctx; j += 256) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
+    for (int j = j0 + threadIdx.x; j < ctx; j += 256) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
     sum = block_sum<256>(sum, red);                     // (its barriers also publish the weights)
     if (a.sink) sum += expf(a.sink[h] - mx);
     const float inv = 1.0f / sum;
     // values: column c by lanes, keys split over the 256 / CW groups
-    float *part = sc + ctx;
+    float *part = sc + ctx;                             // (behind the last score)
     const int64_t vld = a.vld ? a.vld : a.Dv;           // (values inside the key rows: the latent of latent attention)
     for (int cb = 0; cb < a.Dv; cb += 64) {
         const int c = cb + (threadIdx.x & 63), grp = threadIdx.x >> 6;
         float acc = 0.f;
         if (c < a.Dv)
-            for (int j = grp; j < ctx; j += 4) {
+            for (int j = j0 + grp; j < ctx; j += 4) {
                 const int64_t row = (int64_t)bt[j / b.block_size] * b.block_size + j % b.block_size;
                 acc += sc[j] * ld_f(vc, (row * a.G + kvh) * vld + c);
             }
@@ -276,7 +279,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __global__ __launch_bounds__(256) void penalty_table_kernel(const float *__restrict__ r1, const float *__restrict__ r2, int H, int n, float *__restrict__ tab) {
     const int d = blockIdx.x * 256 + threadIdx.x, h = blockIdx.y;
-    if (d < n) tab[(int64_t)h * n + d] = r1[h] * log1pf(r2[h] * (float)d) * kLog2e;
+    if (d < n) tab[(int64_t)h * n + d] = (r2 ? r1[h] * log1pf(r2[h] * (float)d) : r1[h] * (float)d) * kLog2e;      // (r2 null: linear in the distance)
 }
 
 template <int C>
@@ -324,6 +327,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
     const int p0 = st + lr0;                            // first position of the tile
     const int nkeys = p0 + npos;                        // keys the tile's last position sees
     const int ntl = (nkeys + KT - 1) / KT;
+    const int kt0 = a.window > 0 ? max(p0 - a.window + 1, 0) / KT : 0;      // first key tile the tile's first position can see
     const int kch = D >> 3;
     uint4 kreg[NCH], vreg[NCH];
     // a thread's pieces: key skey, 16-byte pieces sch, sch + 4, ... of its row; key group vkg, columns vcl, vcl + 32, ... (one block-table lookup each per tile)
@@ -342,8 +346,8 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
             else if (jk < nkeys && sch + 4 * x < (Dv >> 3)) vreg[x] = *reinterpret_cast<const uint4 *>(vrow + (sch + 4 * x) * 8);
         }
     };
-    if (z < ntl) request(z * KT);
-    for (int kt = z; kt < ntl; kt += nsplit) {
+    if (kt0 + z < ntl) request((kt0 + z) * KT);
+    for (int kt = kt0 + z; kt < ntl; kt += nsplit) {
         const int k0 = kt * KT;
         const int dmin = max(p0 - (k0 + KT - 1), 0);    // smallest distance a visible key of this tile can have
         __syncthreads();
@@ -385,7 +389,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
                     const int dist = pos[i] - j;
                     float v = s[nt][i] * scale2;
                     if (a.pen) v -= pen[(hgi[i] << 7) + min(max(dist - dmin, 0), 127)];
-                    v = dist < 0 ? -INFINITY : v;
+                    v = (dist < 0 || (a.window > 0 && dist >= a.window)) ? -INFINITY : v;
                     s[nt][i] = v;
                     mx[i] = fmaxf(mx[i], v);
                 }
@@ -479,7 +483,9 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
     const int c = cb + (threadIdx.x & 31), part = threadIdx.x >> 5;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0, st = b.start[sq];
     const int D = a.D, Dv = a.Dv, half = a.rot_dims / 2;
-    const float dec = GATED ? 0.f : a.decay[h];
+    const bool tok = !GATED && a.tok_gate != nullptr;     // (keep, take) per token and head instead of decay[h]
+    const float dec = (GATED || tok) ? 0.f : a.decay[h];
+    const int Dr = Dv - a.v_ones;                          // value columns that proj holds; the rest are ones
     float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
     const bool live = c < Dv;
     float s[RMAX];
@@ -487,6 +493,7 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
     for (int r = 0; r < RMAX; ++r) { const int d = part + r * 8; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; }
     for (int i = 0; i < n; ++i) {
         const int t = r0 + i, buf = i & 1;
+        const float keep = tok ? a.tok_gate[((int64_t)t * a.H + h) * 2] : dec, take = tok ? a.tok_gate[((int64_t)t * a.H + h) * 2 + 1] : 1.f;
         const PT *pr = (const PT *)a.proj + (int64_t)t * a.ld;
         const PT *q = pr + a.qcol + (int64_t)h * D, *k = pr + a.kcol + (int64_t)h * D;
         for (int d = threadIdx.x; d < D; d += 256) {
@@ -502,15 +509,16 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
                 qv *= a.qscale;
                 as[buf][d] = expf(log_sigmoid(ld_f((const PT *)a.az, (int64_t)t * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d]) * a.inv_tau);
             }
+            if (tok) { qv *= a.qscale; kv *= take; }
             qs[buf][d] = qv; ks[buf][d] = kv * a.kscale;
         }
         __syncthreads();
-        const float v = live ? ld_f(pr, a.vcol + (int64_t)h * Dv + c) : 0.f;
+        const float v = live ? (c < Dr ? ld_f(pr, a.vcol + (int64_t)h * Dr + c) : 1.f) : 0.f;
         float o = 0.f;
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
             const int d = part + r * 8;
-            if (d < D) { s[r] = (GATED ? as[buf][d] : dec) * s[r] + ks[buf][d] * v; o += s[r] * qs[buf][d]; }
+            if (d < D) { s[r] = (GATED ? as[buf][d] : keep) * s[r] + ks[buf][d] * v; o += s[r] * qs[buf][d]; }
         }
         red[part][threadIdx.x & 31] = o;
         __syncthreads();
@@ -538,11 +546,13 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
     extern __shared__ float rsm[];
     const int D = a.D, Dv = a.Dv, half = a.rot_dims / 2;
     float *qs = rsm, *ks = qs + TB * D, *vs = ks + TB * D, *partial = vs + TB * 32;      // [TB][D], [TB][D], [TB][32], [TB][8][32]
-    float *as = partial + TB * 8 * 32;                                                    // GATED: [TB][D] decays
+    float *as = partial + TB * 8 * 32;                                                    // GATED: [TB][D] decays; token-gated: [TB] keep, [TB] take
     const int sq = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * 32;
     const int cl = threadIdx.x & 31, c = cb + cl, part = threadIdx.x >> 5;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0, st = b.start[sq];
-    const float dec = GATED ? 0.f : a.decay[h];
+    const bool tok = !GATED && a.tok_gate != nullptr;
+    const float dec = (GATED || tok) ? 0.f : a.decay[h];
+    const int Dr = Dv - a.v_ones;
     float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
     const bool live = c < Dv;
     float s[RMAX];
@@ -551,9 +561,13 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
     for (int i0 = 0; i0 < n; i0 += TB) {
         const int nb = min(TB, n - i0);
         __syncthreads();
+        if (tok) {
+            if (threadIdx.x < 2 * nb) as[(threadIdx.x & 1) * TB + (threadIdx.x >> 1)] = a.tok_gate[((int64_t)(r0 + i0 + (threadIdx.x >> 1)) * a.H + h) * 2 + (threadIdx.x & 1)];
+            __syncthreads();
+        }
         const int dsh = (D & (D - 1)) == 0 ? 31 - __clz(D) : -1;
         // fully rotated bf16 heads: a thread takes 8 coordinates of the lower half and their partners of the upper half as 16-byte loads
-        const bool fast = !GATED && sizeof(PT) == 2 && a.rot_dims == D && (half & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol) & 7) == 0 && ((uintptr_t)a.proj & 15) == 0;
+        const bool fast = !GATED && !tok && sizeof(PT) == 2 && a.rot_dims == D && (half & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol) & 7) == 0 && ((uintptr_t)a.proj & 15) == 0;
         if (fast) {
             const int cpt = half >> 3;                                   // 8-coordinate pieces of a half
             for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
@@ -591,6 +605,18 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                     as[i * D + d0 + y] = exp2f(-a.inv_tau * __log2f(1.0f + exp2f(-kLog2e * (ld_f(ze, y) + bp[y]))));
                 }
             }
+        } else if (tok && sizeof(PT) == 2 && a.rot_dims == 0 && (D & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol) & 7) == 0 && ((uintptr_t)a.proj & 15) == 0) {
+            // token-gated, 16-bit rows: 8 consecutive channels of one token as 16-byte loads; the token's input gate rides on its key
+            const int cpt = D >> 3;
+            for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
+                const int i = idx / cpt, d0 = (idx - i * cpt) << 3;
+                const bf16_t *pr = (const bf16_t *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
+                const uint4 qv = *reinterpret_cast<const uint4 *>(pr + a.qcol + (int64_t)h * D + d0), kv = *reinterpret_cast<const uint4 *>(pr + a.kcol + (int64_t)h * D + d0);
+                const bf16_t *qe = reinterpret_cast<const bf16_t *>(&qv), *ke = reinterpret_cast<const bf16_t *>(&kv);
+                const float take = as[TB + i];
+#pragma unroll
+                for (int y = 0; y < 8; ++y) { qs[i * D + d0 + y] = ld_f(qe, y) * a.qscale; ks[i * D + d0 + y] = ld_f(ke, y) * take * a.kscale; }
+            }
         } else
         for (int idx = threadIdx.x; idx < nb * D; idx += 256) {
             const int i = dsh >= 0 ? idx >> dsh : idx / D, d = idx - i * D;
@@ -608,11 +634,12 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                 qv *= a.qscale;
                 as[idx] = expf(log_sigmoid(ld_f((const PT *)a.az, (int64_t)(r0 + i0 + i) * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d]) * a.inv_tau);
             }
+            if (tok) { qv *= a.qscale; kv *= as[TB + i]; }
             qs[idx] = qv; ks[idx] = kv * a.kscale;
         }
         for (int idx = threadIdx.x; idx < nb * 32; idx += 256) {
             const int i = idx >> 5, cc = cb + (idx & 31);
-            vs[idx] = cc < Dv ? ld_f((const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld, a.vcol + (int64_t)h * Dv + cc) : 0.f;
+            vs[idx] = cc < Dv ? (cc < Dr ? ld_f((const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld, a.vcol + (int64_t)h * Dr + cc) : 1.f) : 0.f;
         }
         __syncthreads();
         for (int i = 0; i < nb; ++i) {
@@ -637,6 +664,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                         if (part * RMAX + r < D) { s[r] = ar[r] * s[r] + kr[r] * v; o += s[r] * qr[r]; }
                 }
             } else if (D == 8 * RMAX) {
+                const float dd = tok ? as[i] : dec;
                 float kk[RMAX], qq[RMAX];
 #pragma unroll
                 for (int r = 0; r < RMAX; r += 4) {
@@ -644,11 +672,12 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                     *reinterpret_cast<float4 *>(qq + r) = *reinterpret_cast<const float4 *>(qr + r);
                 }
 #pragma unroll
-                for (int r = 0; r < RMAX; ++r) { s[r] = dec * s[r] + kk[r] * v; o += s[r] * qq[r]; }
+                for (int r = 0; r < RMAX; ++r) { s[r] = dd * s[r] + kk[r] * v; o += s[r] * qq[r]; }
             } else {
+                const float dd = tok ? as[i] : dec;
 #pragma unroll
                 for (int r = 0; r < RMAX; ++r)
-                    if (part * RMAX + r < D) { s[r] = dec * s[r] + kr[r] * v; o += s[r] * qr[r]; }
+                    if (part * RMAX + r < D) { s[r] = dd * s[r] + kr[r] * v; o += s[r] * qr[r]; }
             }
             partial[(i * 8 + part) * 32 + cl] = o;
         }
@@ -836,12 +865,19 @@ int penalty_table(const float *r1, const float *r2, int64_t H, int64_t n, float 
     penalty_table_kernel<<<dim3((unsigned)((n + 255) / 256), (unsigned)H), dim3(256), 0, s>>>(r1, r2, (int)H, (int)n, tab);
     return launched("penalty_table");
 }
+int linear_penalty_table(const float *slope, int64_t H, int64_t n, float *tab, hipStream_t s) {
+    if (H * n == 0) return 0;
+    penalty_table_kernel<<<dim3((unsigned)((n + 255) / 256), (unsigned)H), dim3(256), 0, s>>>(slope, nullptr, (int)H, (int)n, tab);
+    return launched("linear_penalty_table");
+}
 
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s) {
     if (b.T == 0) return 0;
     if (a.G < 1 || a.H % a.G) return nvr::fail(NVR_ERR_INVALID_ARG, "sink_attention: %d heads over %d key/value heads", a.H, a.G);
-    const size_t lds = ((size_t)a.D + (size_t)b.max_ctx + 256) * 4;
-    if (lds > kMaxLds) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention: a context of %d keys does not fit the score buffer", b.max_ctx);
+    if ((a.r1 || a.r2) && a.slope) return nvr::fail(NVR_ERR_INVALID_ARG, "sink_attention: a logarithmic and a linear penalty together");
+    const size_t keys = a.window > 0 ? (size_t)std::min(b.max_ctx, a.window) : (size_t)b.max_ctx;
+    const size_t lds = ((size_t)a.D + keys + 256) * 4;
+    if (lds > kMaxLds) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention: %zu visible keys do not fit the score buffer", keys);
     const dim3 grid((unsigned)b.T, (unsigned)a.H);
     if (bf16) sink_attn_rows_kernel<bf16_t><<<grid, dim3(256), lds, s>>>(a, b);
     else sink_attn_rows_kernel<float><<<grid, dim3(256), lds, s>>>(a, b);
@@ -856,6 +892,9 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
     const int rows = (a.D + 7) / 8;
     const bool gated = a.az != nullptr;
     if (gated && !a.abias) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: gated decays need their bias");
+    if (gated && a.tok_gate) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: decays per channel and gates per token together");
+    if (a.v_ones < 0 || a.v_ones >= a.Dv) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: %d of %d value columns are ones", a.v_ones, a.Dv);
+    if (!gated && !a.tok_gate && !a.decay) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: no decay");
 #define NVR_RET(R_)                                                                                  \
     do {                                                                                             \
         if (gated) { if (bf16) retention_seq_kernel<R_, bf16_t, true><<<grid, dim3(256), 0, s>>>(a, b);   \
@@ -863,7 +902,7 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
         else if (bf16) retention_seq_kernel<R_, bf16_t, false><<<grid, dim3(256), 0, s>>>(a, b);     \
         else retention_seq_kernel<R_, float, false><<<grid, dim3(256), 0, s>>>(a, b);                \
     } while (0)
-    const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32) * 4;
+    const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32 + 32) * 4;
     if (a.D <= 256 && lds <= 64 * 1024) {                 // (beyond: the token-by-token form, whose LDS does not grow with the key size)
 #define NVR_RETB(R_)                                                                                 \
     do {                                                                                             \

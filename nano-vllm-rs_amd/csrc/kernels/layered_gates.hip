@@ -1,0 +1,283 @@
+// layered_gates.hip — blocks of pre-norm layers with a layer scale (kernels/layered.h): learned positions, the exponential gates and the read-out of a
+// matrix memory (its recurrence is retention's token-gated form, layered.hip), queries / keys / values normed over their projections on their way into the
+// pages, an elementwise gated recurrence, the residual joins.  Norms, gates, states and the residual sum are f32 in both operand types.  wave64, gfx950.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <algorithm>
+#include "../common.h"
+#include "layered.h"
+
+namespace nvr { namespace kl {
+
+namespace {
+
+typedef uint16_t bf16_t;
+__device__ __forceinline__ float ld_f(const float *p, int64_t i) { return p[i]; }
+__device__ __forceinline__ float ld_f(const bf16_t *p, int64_t i) { return __uint_as_float((uint32_t)p[i] << 16); }
+__device__ __forceinline__ void st_f(float *p, int64_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void st_f(bf16_t *p, int64_t i, float v) {       // round to nearest even
+    uint32_t u = __float_as_uint(v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) { p[i] = (bf16_t)((u >> 16) | 0x40); return; }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    p[i] = (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+// sum over the 256 threads of a workgroup; red: 4 floats of LDS; every thread gets the sum
+__device__ __forceinline__ float block_sum(float v, float *red) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+int launched(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return nvr::fail(NVR_ERR_HIP, "%s launch failed: %s", what, hipGetErrorString(e));
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------ embedding with learned positions
+template <class ET>
+__global__ __launch_bounds__(256) void embed_pos_kernel(const ET *__restrict__ E, const ET *__restrict__ P, Batch b, int W, float scale, float *__restrict__ x) {
+    const int t = blockIdx.x, sq = b.row_seq[t];
+    const int64_t p = b.start[sq] + (t - b.cu[sq]);
+    const ET *e = E + b.ids[t] * (int64_t)W;
+    float *xr = x + (int64_t)t * W;
+    for (int c = threadIdx.x; c < W; c += 256) xr[c] = ld_f(e, c) * scale + (P ? ld_f(P, p * W + c) : 0.f);
+}
+
+// ------------------------------------------------------------------------------------------------ exponential gates of a matrix memory
+// One thread per (sequence, head) walks the sequence's rows in order: the running maximum is a scalar recurrence.
+__global__ __launch_bounds__(64) void exp_gates_kernel(const float *__restrict__ pre, int64_t ldp, const float *__restrict__ bi, const float *__restrict__ bfg, float cap, Batch b, int H,
+                                                       float *__restrict__ mstate, float *__restrict__ tok_gate, float *__restrict__ floor_out) {
+    const int sq = blockIdx.x, h = blockIdx.y * 64 + threadIdx.x;
+    if (h >= H) return;
+    const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0;
+    float *ms = mstate + (int64_t)b.slot[sq] * H + h;
+    float m = b.start[sq] > 0 ? *ms : 0.f;
+    const float vbi = bi[h], vbf = bfg[h], icap = 1.0f / cap;
+    for (int i = 0; i < n; ++i) {
+        const int64_t t = r0 + i;
+        const float gi = cap * tanhf((pre[t * ldp + h] + vbi) * icap);
+        const float gf = log_sigmoid_f(cap * tanhf((pre[t * ldp + H + h] + vbf) * icap));
+        const float mn = fmaxf(gf + m, gi);
+        tok_gate[(t * H + h) * 2] = expf(gf + m - mn);
+        tok_gate[(t * H + h) * 2 + 1] = expf(gi - mn);
+        floor_out[t * H + h] = expf(-mn);
+        m = mn;
+    }
+    *ms = m;
+}
+
+// one wave per (row, head)
+template <class OT>
+__global__ __launch_bounds__(256) void memory_readout_kernel(const float *__restrict__ o, const float *__restrict__ floor_in, const OT *__restrict__ gate, int64_t ldg, int64_t gcol, int H,
+                                                             int Dv, float eps, const float *__restrict__ w, OT *__restrict__ out, int64_t ldo) {
+    const int64_t t = blockIdx.x;
+    const int h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (h >= H) return;
+    const float *r = o + (t * H + h) * (int64_t)(Dv + 1);
+    const float inv_den = 1.0f / (fmaxf(fabsf(r[Dv]), floor_in[t * H + h]) + 1e-6f);
+    float ss = 0.f;
+    for (int c = lane; c < Dv; c += 64) { const float v = r[c] * inv_den; ss += v * v; }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
+    for (int c = lane; c < Dv; c += 64) {
+        const int64_t col = (int64_t)h * Dv + c;
+        st_f(out, t * ldo + col, r[c] * inv_den * inv * w[col] * sigmoid_f(ld_f(gate, t * ldg + gcol + col)));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ normed queries, keys and values
+template <class CT>
+__global__ __launch_bounds__(256) void qkv_norm_store_kernel(QkvNormArgs a, Batch b) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, sq = b.row_seq[t];
+    const int p = b.start[sq] + (t - b.cu[sq]);
+    const int blk = b.block_tables[(int64_t)sq * b.max_blocks + p / b.block_size], jj = p % b.block_size;
+    const int64_t row = (int64_t)blk * b.block_size + jj;
+    CT *pr = (CT *)a.proj + (int64_t)t * a.ld;
+    const int qn = a.H * a.D, kn = a.G * a.D;
+    if (a.wq) {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < qn; c += 256) { const float v = ld_f(pr, a.qcol + c); ss += v * v; }
+        float f = 1.0f / sqrtf(block_sum(ss, red) / (float)qn + a.eps);
+        if (a.temp_every > 0) f *= 1.0f + a.temp_coef * logf((float)((p + 1) / a.temp_every) + 1.0f);
+        for (int c = threadIdx.x; c < qn; c += 256) st_f(pr, a.qcol + c, ld_f(pr, a.qcol + c) * f * a.wq[c]);
+    }
+    CT *kd = (CT *)a.kc + row * kn;
+    if (a.wk) {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < kn; c += 256) { const float v = ld_f(pr, a.kcol + c); ss += v * v; }
+        const float f = 1.0f / sqrtf(block_sum(ss, red) / (float)kn + a.eps);
+        for (int c = threadIdx.x; c < kn; c += 256) st_f(kd, c, ld_f(pr, a.kcol + c) * f * a.wk[c]);
+    } else
+        for (int c = threadIdx.x; c < kn; c += 256) kd[c] = pr[a.kcol + c];
+    // values: a wave per key/value head
+    const int lane = threadIdx.x & 63, Dv = a.Dv;
+    CT *vc = (CT *)a.vc;
+    const int64_t grp = ((int64_t)blk * (b.block_size >> 3) + (jj >> 3)) * a.G * Dv;      // grouped pages: [block][block_size / 8][G][Dv][8 keys]
+    for (int g = threadIdx.x >> 6; g < a.G; g += 4) {
+        float f = 1.f;
+        if (a.v_unit) {
+            float ss = 0.f;
+            for (int c = lane; c < Dv; c += 64) { const float v = ld_f(pr, a.vcol + g * Dv + c); ss += v * v; }
+            f = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + a.eps);
+        }
+        for (int c = lane; c < Dv; c += 64) {
+            const float v = ld_f(pr, a.vcol + g * Dv + c) * f;
+            if (a.v_grouped) st_f(vc, (grp + g * Dv + c) * 8 + (jj & 7), v);
+            else st_f(vc, (row * a.G + g) * Dv + c, v);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ elementwise gated recurrence
+// One thread per (sequence, channel); the rows of a sequence in order, eight at a time in flight (the loads do not depend on the recurrence).
+template <class CT>
+__global__ __launch_bounds__(256) void gated_unit_kernel(const CT *__restrict__ proj, int64_t ld, int64_t zcol, int64_t ucol, int64_t gcol, const float *__restrict__ bz,
+                                                         const float *__restrict__ bu, Batch b, int N, float *__restrict__ state, CT *__restrict__ out, int64_t ldo) {
+    const int sq = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= N) return;
+    const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0;
+    float *sp = state + (int64_t)b.slot[sq] * N + c;
+    float S = b.start[sq] > 0 ? *sp : 0.f;
+    const float vbz = bz[c], vbu = bu[c];
+    constexpr int U = 8;
+    for (int i0 = 0; i0 < n; i0 += U) {
+        float z[U], u[U], g[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            const int64_t t = r0 + min(i0 + k, n - 1);
+            z[k] = ld_f(proj, t * ld + zcol + c); u[k] = ld_f(proj, t * ld + ucol + c); g[k] = ld_f(proj, t * ld + gcol + c);
+        }
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            if (i0 + k < n) {
+                const float zz = sigmoid_f(z[k] + vbz), uu = u[k] + vbu;
+                const float cand = uu >= 0.f ? uu + 0.5f : sigmoid_f(uu);
+                S = (1.0f - zz) * S + zz * cand;
+                st_f(out, (int64_t)(r0 + i0 + k) * ldo + c, S * (g[k] * sigmoid_f(g[k])));
+            }
+        }
+    }
+    *sp = S;
+}
+
+// ------------------------------------------------------------------------------------------------ residual joins
+// One workgroup per row.
+template <class YT, bool TWO>
+__global__ __launch_bounds__(256) void residual_join_kernel(JoinArgs a) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    const int W = (int)a.W;
+    float *xr = a.x + t * W;
+    const YT *y1 = (const YT *)a.y1 + t * a.ld1, *y2 = TWO ? (const YT *)a.y2 + t * a.ld2 : nullptr;
+    float f1 = 1.f, f2 = 1.f;
+    if (TWO) {
+        float s1 = 0.f, s2 = 0.f;
+        for (int c = threadIdx.x; c < W; c += 256) { const float u = ld_f(y1, c), v = ld_f(y2, c); s1 += u * u; s2 += v * v; }
+        f1 = 1.0f / sqrtf(block_sum(s1, red) / (float)W + a.eps);
+        f2 = 1.0f / sqrtf(block_sum(s2, red) / (float)W + a.eps);
+    }
+    float sn = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float r = ld_f(y1, c);
+        if (TWO) r = 0.5f * (r * f1 * a.w1[c] + ld_f(y2, c) * f2 * a.w2[c]);
+        const float v = xr[c] + (a.ls ? a.ls[c] * r : r);
+        xr[c] = v; sn += v * v;
+    }
+    if (a.wn) {
+        const float fn = 1.0f / sqrtf(block_sum(sn, red) / (float)W + a.eps);
+        YT *o = (YT *)a.out + t * a.ldo;
+        for (int c = threadIdx.x; c < W; c += 256) st_f(o, c, xr[c] * fn * a.wn[c]);      // (a thread re-reads what it wrote)
+    }
+}
+
+template <class CT>
+__global__ __launch_bounds__(256) void relu_squared_kernel(const CT *__restrict__ z, int64_t ldz, int64_t T, int64_t F, CT *__restrict__ out, int64_t ldo) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= T * F) return;
+    const int64_t t = i / F, c = i - t * F;
+    const float v = fmaxf(ld_f(z, t * ldz + c), 0.f);
+    st_f(out, t * ldo + c, v * v);
+}
+
+__global__ __launch_bounds__(256) void scale_f32_kernel(float *__restrict__ y, int64_t n, float c) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] *= c;
+}
+
+}  // namespace
+
+int embed_pos(const void *E, const void *P, bool bf16, const Batch &b, int64_t W, float scale, float *x, hipStream_t s) {
+    if (b.T == 0) return 0;
+    if (bf16) embed_pos_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)E, (const bf16_t *)P, b, (int)W, scale, x);
+    else embed_pos_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const float *)E, (const float *)P, b, (int)W, scale, x);
+    return launched("embed_pos");
+}
+
+int exp_gates(const float *pre, int64_t ldp, const float *bi, const float *bf, float cap, const Batch &b, int64_t H, float *mstate, float *tok_gate, float *floor_out,
+              hipStream_t s) {
+    if (b.T == 0) return 0;
+    if (!(cap > 0.f)) return nvr::fail(NVR_ERR_INVALID_ARG, "exp_gates: the gates' cap must be positive");
+    exp_gates_kernel<<<dim3((unsigned)b.B, (unsigned)((H + 63) / 64)), dim3(64), 0, s>>>(pre, ldp, bi, bf, cap, b, (int)H, mstate, tok_gate, floor_out);
+    return launched("exp_gates");
+}
+
+int memory_readout(const float *o, const float *floor_in, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, const float *w, void *out,
+                   int64_t ldo, bool bf16, hipStream_t s) {
+    if (T == 0) return 0;
+    const dim3 grid((unsigned)T, (unsigned)((H + 3) / 4));
+    if (bf16) memory_readout_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(o, floor_in, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (bf16_t *)out, ldo);
+    else memory_readout_kernel<float><<<grid, dim3(256), 0, s>>>(o, floor_in, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (float *)out, ldo);
+    return launched("memory_readout");
+}
+
+int qkv_norm_store(const QkvNormArgs &a, const Batch &b, bool bf16, hipStream_t s) {
+    if (b.T == 0) return 0;
+    if (a.v_grouped && b.block_size % 8) return nvr::fail(NVR_ERR_INVALID_ARG, "qkv_norm_store: grouped value pages need pages of a multiple of 8 tokens");
+    if (bf16) qkv_norm_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
+    else qkv_norm_store_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
+    return launched("qkv_norm_store");
+}
+
+int gated_unit(const void *proj, int64_t ld, int64_t zcol, int64_t ucol, int64_t gcol, const float *bz, const float *bu, const Batch &b, int64_t N, float *state, void *out, int64_t ldo,
+               bool bf16, hipStream_t s) {
+    if (b.T == 0 || N == 0) return 0;
+    const dim3 grid((unsigned)((N + 255) / 256), (unsigned)b.B);
+    if (bf16) gated_unit_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)proj, ld, zcol, ucol, gcol, bz, bu, b, (int)N, state, (bf16_t *)out, ldo);
+    else gated_unit_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)proj, ld, zcol, ucol, gcol, bz, bu, b, (int)N, state, (float *)out, ldo);
+    return launched("gated_unit");
+}
+
+int residual_join(const JoinArgs &a, bool bf16, hipStream_t s) {
+    if (a.T == 0) return 0;
+    if (a.y2 && (!a.w1 || !a.w2)) return nvr::fail(NVR_ERR_INVALID_ARG, "residual_join: two branches need their norms' weights");
+    const dim3 grid((unsigned)a.T);
+    if (a.y2) { if (bf16) residual_join_kernel<bf16_t, true><<<grid, dim3(256), 0, s>>>(a); else residual_join_kernel<float, true><<<grid, dim3(256), 0, s>>>(a); }
+    else { if (bf16) residual_join_kernel<bf16_t, false><<<grid, dim3(256), 0, s>>>(a); else residual_join_kernel<float, false><<<grid, dim3(256), 0, s>>>(a); }
+    return launched("residual_join");
+}
+
+int relu_squared(const void *z, int64_t ldz, int64_t T, int64_t F, void *out, int64_t ldo, bool bf16, hipStream_t s) {
+    if (T * F == 0) return 0;
+    const dim3 grid((unsigned)((T * F + 255) / 256));
+    if (bf16) relu_squared_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)z, ldz, T, F, (bf16_t *)out, ldo);
+    else relu_squared_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)z, ldz, T, F, (float *)out, ldo);
+    return launched("relu_squared");
+}
+
+int scale_f32(float *y, int64_t n, float c, hipStream_t s) {
+    if (n == 0) return 0;
+    scale_f32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(y, n, c);
+    return launched("scale_f32");
+}
+
+}}  // namespace nvr::kl

@@ -67,6 +67,7 @@ int LayeredModel::init(nvr_model_runner &r) {
     r.Hd = W; r.V = r.Vl = V; r.vocab_start = 0; r.L = (int64_t)spec.runs.size();
     r.block_size = (int64_t)r.cfg.kvcache_block_size; r.max_tokens = (int64_t)r.cfg.max_num_batched_tokens; r.max_seqs = (int64_t)r.cfg.max_num_seqs;
     r.max_pos = std::max<int64_t>((int64_t)r.cfg.max_model_len, 1);
+    if (spec.max_positions > 0) r.max_pos = std::min(r.max_pos, spec.max_positions);     // (learned positions: the table ends there)
     r.max_blocks_per_seq = (r.max_pos + r.block_size - 1) / r.block_size + 1;
     slots = r.cfg.num_state_slots ? (int64_t)r.cfg.num_state_slots : r.max_seqs;
     slot_par.assign((size_t)slots, 0);
@@ -79,6 +80,7 @@ int LayeredModel::init(nvr_model_runner &r) {
     { int v = 0; if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, r.device) == hipSuccess && v > 0) r.num_cus = v; }
 
     if (spec.layout == LayeredSpec::SEQUENTIAL) RC(init_sequential(r));
+    else if (spec.layout == LayeredSpec::SCALED) RC(init_scaled(r));
     else {
     // weights (zero until loaded)
     const int64_t taps = spec.taps;
@@ -208,6 +210,7 @@ int LayeredModel::load_tensor(nvr_model_runner &r, const char *name_in, int dtyp
     if (dtype < 0 || dtype > 2) return fail(NVR_ERR_INVALID_ARG, "load_tensor: dtype %d", dtype);
     const std::string name(name_in);
     if (spec.layout == LayeredSpec::SEQUENTIAL) return load_sequential(r, name, dtype, shape, ndim, data);
+    if (spec.layout == LayeredSpec::SCALED) return load_scaled(r, name, dtype, shape, ndim, data);
     const int64_t W = spec.width, V = spec.vocab;
     auto is2 = [&](int64_t a, int64_t b) { return ndim == 2 && shape[0] == a && shape[1] == b; };
     auto bad = [&]() { return fail(NVR_ERR_LEN_MISMATCH, "load_tensor: '%s' has the wrong shape", name_in); };
@@ -391,6 +394,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
 
 int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
     if (spec.layout == LayeredSpec::SEQUENTIAL) return forward_sequential(r, p);
+    if (spec.layout == LayeredSpec::SCALED) return forward_scaled(r, p);
     const kl::Batch &b = p.b;
     const int32_t *d_want = p.d_want;
     const int64_t T = p.T, R = p.R, max_ctx = p.max_ctx;
@@ -811,6 +815,247 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
     kl::GroupNormArgs n{}; n.in = x; n.ldi = W; n.in_f32 = true; n.rows = p.d_want; n.rows_n = R; n.W = W; n.groups = groups; n.eps = eps; n.w = wfinal; n.out = xsel; n.ldo = W;
     RC(kl::group_norm(n, bf16, s));
     return gemm(r, xsel, W, head, R, W, spec.vocab, r.logits, true);
+}
+
+// ===================================================================================================================================================
+// Scaled layout: x <- x + ls1 * mixer(n1(x)); x <- x + ls2 * ff(n2(x)); learned positions; a layer run uses the weights of layer spec.runs[run] and a
+// cache / state of its own.
+
+namespace { inline int64_t pad16(int64_t n) { return (n + 15) / 16 * 16; } }
+
+int LayeredModel::init_scaled(nvr_model_runner &r) {
+    const int64_t W = spec.width, V = spec.vocab, MT = r.max_tokens;
+    auto named = [&](void **p, size_t bytes) {              // (the buffers the destructor frees by name)
+        RC(dmalloc((char **)p, bytes));
+        NVR_HIP_CHECK(hipMemset(*p, 0, bytes ? bytes : 16));
+        return (int)NVR_OK;
+    };
+    lw.resize(spec.layers.size());
+    int64_t max_nmix = 0, max_hv = 0, max_ro = 0, max_ff = 0, max_gw = 0, max_gpad = 16, max_h = 1;
+    for (size_t i = 0; i < spec.layers.size(); ++i) {
+        const LayeredSpec::Layer &L = spec.layers[i]; LayerW &w = lw[i];
+        if (L.weights_of >= 0) continue;                    // (its runs read the source's LayerW)
+        const int64_t hd = L.heads * L.dim, hv = L.heads * L.vdim;
+        RC(own(&w.n1, (size_t)W * 4)); RC(own(&w.ls1, (size_t)W * 4));
+        if (L.has_mlp) {
+            RC(own(&w.n2, (size_t)W * 4)); RC(own(&w.ls2, (size_t)W * 4));
+            RC(own(&w.up, (size_t)(L.ff * W * esz))); RC(own(&w.down, (size_t)(W * L.ff * esz)));
+            max_ff = std::max(max_ff, L.ff);
+        }
+        if (L.mixer == LayeredSpec::MLSTM) {
+            w.qcol = 0; w.kcol = pad16(hd); w.vcol = w.kcol + pad16(hd); w.gcol = w.vcol + pad16(hv); w.nmix = w.gcol + pad16(hv);
+            w.gpad = pad16(2 * L.heads);
+            RC(own(&w.wgates, (size_t)(w.gpad * W * esz))); RC(own(&w.bi, (size_t)L.heads * 4)); RC(own(&w.bfg, (size_t)L.heads * 4)); RC(own(&w.hnorm, (size_t)hv * 4));
+            max_ro = std::max(max_ro, L.heads * (L.vdim + 1)); max_gpad = std::max(max_gpad, w.gpad); max_h = std::max(max_h, L.heads);
+        } else if (L.mixer == LayeredSpec::ATTN_GRU) {
+            const int64_t kn = L.kv_heads * L.dim, vn = L.kv_heads * L.vdim, gw = L.gru_width;
+            w.qcol = 0; w.kcol = pad16(hd); w.vcol = w.kcol + pad16(kn); w.gcol = w.vcol + pad16(vn); w.zcol = w.gcol + pad16(hv); w.ucol = w.zcol + pad16(gw); w.rgcol = w.ucol + pad16(gw);
+            w.nmix = w.rgcol + pad16(gw);
+            RC(own(&w.qn, (size_t)hd * 4)); RC(own(&w.kn, (size_t)kn * 4)); RC(named((void **)&w.sink, (size_t)L.heads * 4));
+            RC(own(&w.bz, (size_t)gw * 4)); RC(own(&w.bu, (size_t)gw * 4)); RC(own(&w.outl, (size_t)W * 4)); RC(own(&w.outr, (size_t)W * 4));
+            RC(own(&w.wo2, (size_t)(W * gw * esz)));
+            std::vector<float> sl((size_t)L.heads);
+            for (int64_t h = 0; h < L.heads; ++h) sl[(size_t)h] = (float)std::exp2(-8.0 * (double)(h + 1) / (double)L.heads);
+            RC(own(&w.slope, sl.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.slope, sl.data(), sl.size() * 4, hipMemcpyHostToDevice));
+            if (std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) == attn_groups.end()) attn_groups.push_back(L.heads / L.kv_heads);
+            w.flash = bf16 && L.dim == L.vdim && nvr::kb::flash_prefill_ok((int)L.dim, (int)L.heads, (int)L.kv_heads) && hv % 8 == 0;
+            if (w.flash && std::find(flash_groups.begin(), flash_groups.end(), L.heads / L.kv_heads) == flash_groups.end()) flash_groups.push_back(L.heads / L.kv_heads);
+            if (bf16) {                                     // the matrix-core attention takes the slopes as its table of penalties by distance (the window bounds the distance)
+                const int64_t n = std::min<int64_t>(r.max_pos, L.window) + 1;
+                RC(dmalloc(&w.pen, (size_t)(L.heads * n * 4)));
+                RC(kl::linear_penalty_table(w.slope, L.heads, n, w.pen, r.stream)); w.pen_dirty = false;
+            }
+            max_gw = std::max(max_gw, gw);
+        } else return fail(NVR_ERR_UNSUPPORTED, "layer %zu: this mixer does not belong to the scaled layout", i);
+        RC(named(&w.mix, (size_t)(w.nmix * W * esz))); RC(own(&w.wo, (size_t)(W * hv * esz)));
+        max_nmix = std::max(max_nmix, w.nmix); max_hv = std::max(max_hv, hv);
+    }
+    RC(named(&embed, (size_t)(V * W * esz))); RC(named(&head, (size_t)(V * W * esz))); RC(own(&wfinal, (size_t)W * 4));
+    RC(own(&pos, (size_t)(spec.max_positions * W * esz)));
+
+    // pages for every run with attention; per slot the matrix memory (with the column of the keys' running sum and the running maxima) or the recurrence's state
+    size_t block_bytes = 0;
+    for (int li : spec.runs) {
+        const LayeredSpec::Layer &L = spec.layers[(size_t)li];
+        if (L.mixer == LayeredSpec::ATTN_GRU) block_bytes += (size_t)(r.block_size * L.kv_heads * (L.dim + L.vdim) * esz);
+    }
+    if (r.cfg.num_kvcache_blocks >= 0) r.num_blocks = r.cfg.num_kvcache_blocks;
+    else if (r.cfg.num_kvcache_blocks == -1) r.num_blocks = 1000;
+    else {
+        size_t free_b = 0, total_b = 0;
+        NVR_HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+        const double budget = (double)free_b - (1.0 - r.cfg.gpu_memory_utilization) * (double)total_b - (double)(MT * (8 * W + 2 * max_nmix + 2 * max_ro + 4 * max_ff) * 4);
+        const int64_t nb = block_bytes ? (int64_t)(budget * 0.9 / (double)block_bytes) : 1000;
+        if (nb < 1) return fail(NVR_ERR_HIP, "not enough free HBM for one KV block");
+        r.num_blocks = nb;
+    }
+    rs.resize(spec.runs.size());
+    for (size_t ri = 0; ri < spec.runs.size(); ++ri) {
+        const LayeredSpec::Layer &L = spec.layers[(size_t)spec.runs[ri]]; RunState &st = rs[ri];
+        if (L.mixer == LayeredSpec::ATTN_GRU) {
+            RC(named(&st.kc, (size_t)(r.num_blocks * r.block_size * L.kv_heads * L.dim * esz))); RC(named(&st.vc, (size_t)(r.num_blocks * r.block_size * L.kv_heads * L.vdim * esz)));
+            RC(named((void **)&st.state, (size_t)(slots * L.gru_width * 4)));
+        } else {
+            RC(named((void **)&st.state, (size_t)(slots * L.heads * L.dim * (L.vdim + 1) * 4))); RC(own(&st.mstate, (size_t)(slots * L.heads * 4)));
+        }
+    }
+
+    // activations
+    RC(named((void **)&x, (size_t)(MT * W * 4)));
+    RC(named(&a1, (size_t)(MT * W * esz))); RC(named(&a2, (size_t)(MT * W * esz))); RC(named(&tmp, (size_t)(MT * W * esz))); RC(own(&tmp2, (size_t)(MT * W * esz)));
+    RC(named(&proj, (size_t)(MT * max_nmix * esz))); RC(named(&cat, (size_t)(MT * max_hv * esz))); RC(own(&gy, (size_t)(MT * max_gw * esz)));
+    RC(named((void **)&ret_o, (size_t)(MT * max_ro * 4)));
+    RC(own(&gpre, (size_t)(MT * max_gpad * 4))); RC(own(&tokg, (size_t)(MT * max_h * 2 * 4))); RC(own(&gfloor, (size_t)(MT * max_h * 4)));
+    RC(named(&gu, (size_t)(MT * max_ff * esz))); RC(own(&act, (size_t)(MT * max_ff * esz)));
+    return NVR_OK;
+}
+
+// Tensors by the names of the checkpoint: "embed", "pos" [positions][W], "head", "final.norm" [W]; per layer i with tensors of its own "l<i>.norm1" / "norm2" / "ls1" / "ls2" [W],
+// matrix memory "l<i>.mix.{q,k,v,g,o,norm,i,i.b,f,f.b}", side by side "l<i>.mix.left.{q,k,v,g,o,q.norm,k.norm,sink,out}" and "l<i>.mix.right.{z,z.b,x,x.b,g,o,out}",
+// "l<i>.mlp.{up,down}".  Linear weights are [out][in].
+int LayeredModel::load_scaled(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data) {
+    const int64_t W = spec.width, V = spec.vocab, nL = (int64_t)spec.layers.size();
+    const char *name_in = name.c_str();
+    auto is2 = [&](int64_t a, int64_t b) { return ndim == 2 && shape[0] == a && shape[1] == b; };
+    auto bad = [&]() { return fail(NVR_ERR_LEN_MISMATCH, "load_tensor: '%s' has the wrong shape", name_in); };
+    auto unknown = [&]() { return fail(NVR_ERR_UNSUPPORTED, "load_tensor: unknown tensor '%s'", name_in); };
+    auto vec = [&](float *dst, int64_t n) { return (dst && ndim == 1 && shape[0] == n) ? put(r, dst, n, 1, n, dtype, data, false) : bad(); };
+    auto mat = [&](void *dst, int64_t ld, int64_t rows, int64_t cols) { return (dst && is2(rows, cols)) ? put(r, dst, ld, rows, cols, dtype, data, true) : bad(); };
+    auto rows_at = [&](void *base, int64_t row0, int64_t ld) { return (void *)((char *)base + (size_t)(row0 * ld * esz)); };
+    if (name == "embed") return mat(embed, W, V, W);
+    if (name == "head") return mat(head, W, V, W);
+    if (name == "pos") return mat(pos, W, spec.max_positions, W);
+    if (name == "final.norm") return vec(wfinal, W);
+    size_t dot = name.find('.');
+    if (name.size() < 3 || name[0] != 'l' || dot == std::string::npos || dot < 2) return unknown();
+    int64_t li = 0;
+    for (size_t i = 1; i < dot; ++i) { if (name[i] < '0' || name[i] > '9') return unknown(); li = li * 10 + (name[i] - '0'); }
+    if (li >= nL) return fail(NVR_ERR_UNSUPPORTED, "load_tensor: '%s' names a layer the model does not have", name_in);
+    const LayeredSpec::Layer &L = spec.layers[(size_t)li]; LayerW &w = lw[(size_t)li];
+    if (L.weights_of >= 0) return fail(NVR_ERR_UNSUPPORTED, "load_tensor: '%s' names a layer that uses the tensors of layer %ld", name_in, (long)L.weights_of);
+    const std::string rest = name.substr(dot + 1);
+    const int64_t hd = L.heads * L.dim, hv = L.heads * L.vdim;
+    if (rest == "norm1") return vec(w.n1, W);
+    if (rest == "ls1") return vec(w.ls1, W);
+    if (L.has_mlp) {
+        if (rest == "norm2") return vec(w.n2, W);
+        if (rest == "ls2") return vec(w.ls2, W);
+        if (rest == "mlp.up") return mat(w.up, W, L.ff, W);
+        if (rest == "mlp.down") return mat(w.down, L.ff, W, L.ff);
+    }
+    if (L.mixer == LayeredSpec::MLSTM) {
+        if (rest == "mix.q") return mat(rows_at(w.mix, w.qcol, W), W, hd, W);
+        if (rest == "mix.k") return mat(rows_at(w.mix, w.kcol, W), W, hd, W);
+        if (rest == "mix.v") return mat(rows_at(w.mix, w.vcol, W), W, hv, W);
+        if (rest == "mix.g") return mat(rows_at(w.mix, w.gcol, W), W, hv, W);
+        if (rest == "mix.o") return mat(w.wo, hv, W, hv);
+        if (rest == "mix.norm") return vec(w.hnorm, hv);
+        if (rest == "mix.i") return mat(w.wgates, W, L.heads, W);
+        if (rest == "mix.f") return mat(rows_at(w.wgates, L.heads, W), W, L.heads, W);
+        if (rest == "mix.i.b") return vec(w.bi, L.heads);
+        if (rest == "mix.f.b") return vec(w.bfg, L.heads);
+    } else {
+        const int64_t kn = L.kv_heads * L.dim, vn = L.kv_heads * L.vdim, gw = L.gru_width;
+        if (rest == "mix.left.q") return mat(rows_at(w.mix, w.qcol, W), W, hd, W);
+        if (rest == "mix.left.k") return mat(rows_at(w.mix, w.kcol, W), W, kn, W);
+        if (rest == "mix.left.v") return mat(rows_at(w.mix, w.vcol, W), W, vn, W);
+        if (rest == "mix.left.g") return mat(rows_at(w.mix, w.gcol, W), W, hv, W);
+        if (rest == "mix.left.o") return mat(w.wo, hv, W, hv);
+        if (rest == "mix.left.q.norm") return vec(w.qn, hd);
+        if (rest == "mix.left.k.norm") return vec(w.kn, kn);
+        if (rest == "mix.left.sink") return vec(w.sink, L.heads);
+        if (rest == "mix.left.out") return vec(w.outl, W);
+        if (rest == "mix.right.z") return mat(rows_at(w.mix, w.zcol, W), W, gw, W);
+        if (rest == "mix.right.x") return mat(rows_at(w.mix, w.ucol, W), W, gw, W);
+        if (rest == "mix.right.g") return mat(rows_at(w.mix, w.rgcol, W), W, gw, W);
+        if (rest == "mix.right.z.b") return vec(w.bz, gw);
+        if (rest == "mix.right.x.b") return vec(w.bu, gw);
+        if (rest == "mix.right.o") return mat(w.wo2, gw, W, gw);
+        if (rest == "mix.right.out") return vec(w.outr, W);
+    }
+    return unknown();
+}
+
+int LayeredModel::forward_scaled(nvr_model_runner &r, const StepPlan &p) {
+    const kl::Batch &b = p.b;
+    const int64_t T = p.T, R = p.R, W = spec.width, nR = (int64_t)spec.runs.size();
+    const float eps = (float)spec.eps;
+    hipStream_t s = r.stream;
+    auto at = [&](void *base, int64_t col) { return (void *)((char *)base + (size_t)(col * esz)); };
+    RC(kl::embed_pos(embed, pos, bf16, b, W, (float)spec.embedding_scale, x, s));
+    {   // the first layer's input; every later one leaves the join before it
+        kl::GroupNormArgs n{}; n.in = x; n.ldi = W; n.in_f32 = true; n.rows_n = T; n.W = W; n.groups = 1; n.eps = eps; n.w = lw[(size_t)spec.runs[0]].n1; n.out = a1; n.ldo = W;
+        RC(kl::group_norm(n, bf16, s));
+    }
+    for (int64_t ri = 0; ri < nR; ++ri) {
+        const size_t li = (size_t)spec.runs[(size_t)ri];
+        const LayeredSpec::Layer &L = spec.layers[li]; const LayerW &w = lw[li]; RunState &st = rs[(size_t)ri];
+        const int64_t hv = L.heads * L.vdim;
+        const float *next_n1 = ri + 1 < nR ? lw[(size_t)spec.runs[(size_t)ri + 1]].n1 : nullptr;
+        kl::JoinArgs j{}; j.x = x; j.T = T; j.W = W; j.eps = eps; j.ls = w.ls1; j.y1 = tmp; j.ld1 = W;
+        if (L.has_mlp) { j.wn = w.n2; j.out = a2; } else { j.wn = next_n1; j.out = a1; }
+        j.ldo = W;
+        RC(gemm(r, a1, W, w.mix, T, W, w.nmix, proj));
+        if (L.mixer == LayeredSpec::MLSTM) {
+            RC(gemm(r, a1, W, w.wgates, T, W, w.gpad, gpre, true));                  // the gates' pre-activations leave the product in f32
+            RC(kl::exp_gates(gpre, w.gpad, w.bi, w.bfg, (float)L.gate_cap, b, L.heads, st.mstate, tokg, gfloor, s));
+            kl::RetentionArgs a{};
+            a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.rot_dims = 0; a.kscale = 1.0f; a.qscale = 1.0f / std::sqrt((float)L.dim);
+            a.H = (int32_t)L.heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim + 1; a.v_ones = 1; a.tok_gate = tokg; a.state = st.state; a.o = ret_o; a.inv_tau = 1.f;
+            RC(kl::retention(a, b, bf16, s));
+            RC(kl::memory_readout(ret_o, gfloor, proj, w.nmix, w.gcol, T, L.heads, L.vdim, eps, w.hnorm, cat, hv, bf16, s));
+            RC(gemm(r, cat, hv, w.wo, T, hv, W, tmp));
+        } else {
+            kl::SinkAttnArgs a{};
+            a.q = at(proj, w.qcol); a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.sink = w.sink; a.slope = w.slope; a.window = (int32_t)L.window;
+            a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale;
+            a.out = cat; a.ldo = hv;
+            a.v_grouped = w.flash ? 0 : 1;                                           // (a property of the layer: the pages keep one layout)
+            const bool tiled = kl::sink_attention_tiled_ok(a, bf16, (int)r.block_size);
+            kl::QkvNormArgs qa{};
+            qa.proj = proj; qa.ld = w.nmix; qa.qcol = w.qcol; qa.kcol = w.kcol; qa.vcol = w.vcol; qa.H = a.H; qa.G = a.G; qa.D = a.D; qa.Dv = a.Dv; qa.eps = eps;
+            qa.wq = w.qn; qa.wk = w.kn; qa.v_unit = true; qa.temp_coef = (float)L.temp_coef; qa.temp_every = (int32_t)L.temp_every;
+            qa.kc = st.kc; qa.vc = st.vc; qa.v_grouped = tiled && !w.flash;
+            RC(kl::qkv_norm_store(qa, b, bf16, s));
+            if (w.flash && !p.decode_sized) {
+                // prompts and portions: the dense graph's flash kernel in its penalty / sink form, linear in the distance and windowed
+                const size_t gi = (size_t)(std::find(flash_groups.begin(), flash_groups.end(), L.heads / L.kv_heads) - flash_groups.begin());
+                nvr::kt::FlashArgs f{};
+                f.q = (const uint16_t *)a.q; f.ldq = w.nmix; f.k = (const uint16_t *)st.kc; f.v = (const uint16_t *)st.vc; f.ldkv = 0;
+                f.block_tables = b.block_tables; f.max_blocks = b.max_blocks; f.block_size = b.block_size;
+                f.tiles = (const nvr::kt::FlashTile *)(in_dev + p.o_ftiles[gi]); f.ntiles = p.n_ftiles[gi];
+                f.H = (int32_t)L.heads; f.KVH = (int32_t)L.kv_heads; f.D = (int32_t)L.dim; f.scale = (float)L.scale; f.out = (uint16_t *)cat;
+                f.r1 = w.slope; f.r2 = nullptr; f.sink = w.sink; f.ldo = hv; f.window = (int32_t)L.window;
+                RC(nvr::kb::flash_prefill(f, true, s));
+            } else if (tiled) {
+                a.pen = w.pen; a.pen_n = (int32_t)(std::min<int64_t>(r.max_pos, L.window) + 1);
+                const size_t gi = (size_t)(std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) - attn_groups.begin());
+                const int64_t wgs = (int64_t)p.n_tiles[gi] * L.kv_heads, keys = std::min<int64_t>(p.max_ctx, L.window + 64);
+                int64_t nsplit = 1;
+                if (wgs < r.num_cus && keys >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / wgs, (keys + 255) / 256, 16}));
+                RC(kl::sink_attention_tiled(a, b, (const kl::AttnTile *)(in_dev + p.o_tiles[gi]), p.n_tiles[gi], (int)nsplit, attn_ws, attn_ws_bytes, s));
+            } else
+                RC(kl::sink_attention(a, b, bf16, s));
+            RC(kl::sigmoid_gate(cat, hv, at(proj, w.gcol), w.nmix, T, hv, bf16, s));
+            RC(gemm(r, cat, hv, w.wo, T, hv, W, tmp));
+            RC(kl::gated_unit(proj, w.nmix, w.zcol, w.ucol, w.rgcol, w.bz, w.bu, b, L.gru_width, st.state, gy, L.gru_width, bf16, s));
+            RC(gemm(r, gy, L.gru_width, w.wo2, T, L.gru_width, W, tmp2));
+            j.w1 = w.outl; j.y2 = tmp2; j.ld2 = W; j.w2 = w.outr;
+        }
+        RC(kl::residual_join(j, bf16, s));
+        if (L.has_mlp) {
+            RC(gemm(r, a2, W, w.up, T, W, L.ff, gu));
+            RC(kl::relu_squared(gu, L.ff, T, L.ff, act, L.ff, bf16, s));
+            RC(gemm(r, act, L.ff, w.down, T, L.ff, W, tmp));
+            kl::JoinArgs j2{}; j2.x = x; j2.T = T; j2.W = W; j2.eps = eps; j2.ls = w.ls2; j2.y1 = tmp; j2.ld1 = W; j2.wn = next_n1; j2.out = a1; j2.ldo = W;
+            RC(kl::residual_join(j2, bf16, s));
+        }
+    }
+    kl::GroupNormArgs n{}; n.in = x; n.ldi = W; n.in_f32 = true; n.rows = p.d_want; n.rows_n = R; n.W = W; n.groups = 1; n.eps = eps; n.w = wfinal; n.out = xsel; n.ldo = W;
+    RC(kl::group_norm(n, bf16, s));
+    RC(gemm(r, xsel, W, head, R, W, spec.vocab, r.logits, true));
+    if (spec.logit_scale != 1.0) RC(kl::scale_f32(r.logits, R * spec.vocab, (float)spec.logit_scale, s));
+    return NVR_OK;
 }
 
 }  // namespace nvr

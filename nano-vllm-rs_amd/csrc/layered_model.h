@@ -8,6 +8,11 @@
 //                          attention (one cached latent row per token, optionally shared with an earlier layer, optionally with a rotated key part and a
 //                          latent for the queries) or gated linear attention; the feed-forward is dense with a polynomial-norm activation or a mixture of
 //                          experts; a per-layer token input and a weighted average over the outputs of all earlier layers close the layer.
+//   scaled (Sosutar)     — x <- x + ls1 * mixer(n1(x)), then x <- x + ls2 * ff(n2(x)): RMS norms in front, a learned scale per channel behind each sublayer, learned
+//                          positions added to the embedding; the mixer is an exponentially gated matrix memory (mLSTM), or a windowed attention (normed queries, keys
+//                          and values, query temperature, linear distance penalty, sink, output gate) side by side with an elementwise gated recurrence (minGRU),
+//                          each branch normed, half their sum; the feed-forward is dense with a squared ReLU; a layer may use an earlier layer's weights with a
+//                          cache / state of its own (layered_scaled.cpp).
 //
 // The family shares the runner's step interface (sequences with a chunk [start, start + len) each: whole prompts, portions of prompts and
 // single decoded tokens in one batch), the block manager's tables (K/V pages) and state slots (recurrent state, convolution history), the
@@ -26,9 +31,9 @@ struct nvr_model_runner;
 namespace nvr {
 
 struct LayeredSpec {
-    enum Mixer { ATTENTION = 0, RETENTION = 1, LATENT = 2, GLA = 3 };
-    enum Ff { FF_NONE = 0, FF_CLAMPED_GLU = 1, FF_POLY = 2, FF_MOE = 3 };
-    enum Layout { PARALLEL = 0, SEQUENTIAL = 1 };
+    enum Mixer { ATTENTION = 0, RETENTION = 1, LATENT = 2, GLA = 3, MLSTM = 4, ATTN_GRU = 5 };
+    enum Ff { FF_NONE = 0, FF_CLAMPED_GLU = 1, FF_POLY = 2, FF_MOE = 3, FF_RELU2 = 4 };
+    enum Layout { PARALLEL = 0, SEQUENTIAL = 1, SCALED = 2 };
     struct Layer {
         int mixer = ATTENTION;
         int64_t heads = 0, kv_heads = 0, dim = 0, vdim = 0;
@@ -40,6 +45,11 @@ struct LayeredSpec {
         // heads (0: none; rot_base its frequency base), the layer whose cached rows this layer reads (-1: its own), and whether sigmoid(W_g h) gates the heads' output
         int64_t kv_rank = 0, q_rank = 0, rot_dim = 0, kv_from = -1; bool out_gate = false;
         double tau = 1.0;                                   // gated linear attention: decay = sigmoid(z)^(1 / tau)
+        double gate_cap = 0.0;                              // matrix memory: the log gates are cap * tanh(z / cap)
+        int64_t window = 0;                                 // windowed attention: keys less than this many positions back (0: all)
+        double temp_coef = 0.0; int64_t temp_every = 0;     // query temperature 1 + coef ln(floor((p + 1) / every) + 1) (every 0: none)
+        int64_t gru_width = 0;                              // the gated recurrence beside the attention
+        int64_t weights_of = -1;                            // the layer whose tensors this layer uses (-1: its own)
         int ff_kind = FF_NONE;
         int64_t experts = 0, top = 0, expert_ff = 0, shared_ff = 0;   // mixture of experts (shared_ff 0: no shared expert)
     };
@@ -48,12 +58,15 @@ struct LayeredSpec {
     int64_t side_dim = 0;                                   // per-layer token input: numbers per layer and token (0: none)
     int64_t vocab = 0, width = 0;
     double embedding_scale = 1.0, eps = 1e-5, residual_mult = 1.0;
+    int64_t max_positions = 0;                              // learned position vectors (0: none)
+    double logit_scale = 1.0;
     int64_t taps = 1;                                       // causal convolution in front of every sublayer (1: a pointwise gain)
     std::vector<Layer> layers;
     std::vector<int> runs;                                  // layer index of every layer run, in order (loops unrolled)
     bool stateful() const { return true; }                  // convolution history, and recurrent state where there is retention
     static int parse_rugudra(const Json &cfg, LayeredSpec *out);   // (model_registry.cpp)
     static int parse_pusunex(const Json &cfg, LayeredSpec *out);
+    static int parse_sosutar(const Json &cfg, LayeredSpec *out);
 };
 
 class LayeredModel {
@@ -81,8 +94,14 @@ public:
         void *up = nullptr, *down = nullptr; float *act = nullptr;                   // dense feed-forward [ff][W], [W][ff]; 4 coefficients
         float *router = nullptr; void *egu = nullptr, *edown = nullptr, *sgu = nullptr, *sdown = nullptr;   // [E][W] f32; [E][2 f][W]; [E][W][f]; [2 fs][W]; [W][fs]
         void *sgate = nullptr, *sproj = nullptr; float *snorm = nullptr, *dwa = nullptr;   // [side][W], [W][side], [W]; [i + 2]
+        // scaled layout (segments of mix start at multiples of 16 rows)
+        float *ls1 = nullptr, *ls2 = nullptr;                                        // [W] each
+        void *wgates = nullptr; int64_t gpad = 0; float *bi = nullptr, *bfg = nullptr;   // matrix memory: [gpad][W] (input gates' rows, then forget gates'), biases [H]
+        float *qn = nullptr, *kn = nullptr, *slope = nullptr;                        // attention: norm weights over the whole q / k projection; distance slopes [H]
+        int64_t zcol = 0, ucol = 0, rgcol = 0;                                       // gated recurrence: columns of z, x and its gate in the mix projection
+        void *wo2 = nullptr; float *bz = nullptr, *bu = nullptr, *outl = nullptr, *outr = nullptr;   // [W][gru_width]; biases [gru_width]; the branches' norms [W]
     };
-    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; void *rows = nullptr; };   // borrowed: another run's pages (a shared latent)
+    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; void *rows = nullptr; float *mstate = nullptr; };   // mstate: a matrix memory's running maxima [slots][H]   // borrowed: another run's pages (a shared latent)
     std::vector<LayerW> lw;
     std::vector<RunState> rs;
     void *embed = nullptr, *head = nullptr; float gfinal = 1.f;
@@ -92,6 +111,8 @@ public:
     void *qlat = nullptr, *q2 = nullptr, *qabs = nullptr, *ctx = nullptr, *alow = nullptr, *az = nullptr, *act = nullptr, *shared_y = nullptr;
     bool flash_contiguous = false; void *kvx = nullptr;                      // flash tiles refer to rows of the step (not to block tables); expanded keys | values of a step
     int64_t alow_cap = 0; void *side_z = nullptr, *side_g = nullptr;
+    // scaled layout
+    void *pos = nullptr; void *tmp2 = nullptr, *gy = nullptr; float *gpre = nullptr, *tokg = nullptr, *gfloor = nullptr;   // [positions][W]; second branch's output, the recurrence's output; gates
     void *e_x = nullptr;                                                    // experts' inputs gathered in the order of the grouped rows
     void *e_gu = nullptr, *e_act = nullptr, *e_y = nullptr; int32_t *moe_i = nullptr; float *moe_score = nullptr;
     std::vector<void *> owned;                                              // device allocations of the sequential layout (freed with the model)
@@ -123,6 +144,9 @@ private:
     int init_sequential(nvr_model_runner &r);
     int load_sequential(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data);
     int forward_sequential(nvr_model_runner &r, const StepPlan &p);
+    int init_scaled(nvr_model_runner &r);
+    int load_scaled(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data);
+    int forward_scaled(nvr_model_runner &r, const StepPlan &p);
     template <class T> int own(T **p, size_t bytes);
     int gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32 = false);
     int put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t rows, int64_t cols, int dtype, const void *src, bool as_operand);

@@ -60,11 +60,17 @@ int parse_pusunex_spec(const Json &c, nvr_model_spec *out) {
     return LayeredSpec::parse_pusunex(c, &out->layered);
 }
 
+int parse_sosutar_spec(const Json &c, nvr_model_spec *out) {
+    out->family = 1;
+    return LayeredSpec::parse_sosutar(c, &out->layered);
+}
+
 struct Entry { const char *name; int (*parse)(const Json &, nvr_model_spec *); };
 const Entry kRegistry[] = {
     {"Qwen3ForCausalLM", parse_qwen3},
     {"Rugudra", parse_rugudra_spec},
     {"Pusunex", parse_pusunex_spec},
+    {"Sosutar", parse_sosutar_spec},
 };
 
 }  // namespace
@@ -203,6 +209,72 @@ int LayeredSpec::parse_pusunex(const Json &c, LayeredSpec *s) {
         if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
         if (L.heads < 1 || L.dim < 1 || L.vdim < 1) return fail(NVR_ERR_INVALID_ARG, "config: %s heads, dim and vdim must be positive", w.c_str());
         s->layers.push_back(L); s->runs.push_back((int)i);
+    }
+    return NVR_OK;
+}
+
+// Sosutar: x <- x + ls1 * mixer(n1(x)), x <- x + ls2 * ff(n2(x)); learned positions; mixers 'mlstm' (matrix memory with exponential gates capped by gate_cap) and
+// 'parallel' (mixer.left: attention with mask.size, q_temp.{coef, every}, scale; mixer.right: a gated recurrence of 'width' channels); feed-forward 'dense'
+// (squared ReLU) or none; 'weights_of': j gives a layer the tensors of layer j and a cache / state of its own.
+int LayeredSpec::parse_sosutar(const Json &c, LayeredSpec *s) {
+    Reader rd;
+    s->layout = SCALED; s->taps = 1; s->residual_mult = 1.0; s->norm_groups = 1;
+    s->vocab = rd.integer(c, "vocab", ""); s->width = rd.integer(c, "width", "");
+    s->max_positions = rd.integer(c, "max_positions", ""); s->logit_scale = rd.num(c, "logit_scale", "");
+    if (const Json *e = rd.need(c, "embedding", "")) s->embedding_scale = rd.num(*e, "scale", "embedding.");
+    if (const Json *n = rd.need(c, "norm", "")) s->eps = rd.num(*n, "eps", "norm.");
+    const Json *layers = rd.need(c, "layers", "");
+    if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+    if (layers->kind != Json::Arr || layers->arr.empty()) return fail(NVR_ERR_INVALID_ARG, "config: 'layers' is not a list of layers");
+    if (s->vocab < 1 || s->width < 1 || s->max_positions < 1) return fail(NVR_ERR_INVALID_ARG, "config: vocab, width and max_positions must be positive");
+    s->layers.clear(); s->runs.clear();
+    for (size_t i = 0; i < layers->arr.size(); ++i) {
+        const Json &lj = layers->arr[i];
+        const std::string w = "layers[" + std::to_string(i) + "].", wm = w + "mixer.";
+        Layer L;
+        const Json *type = rd.need(lj, "type", w), *mx = rd.need(lj, "mixer", w);
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (type->kind != Json::Str) return fail(NVR_ERR_INVALID_ARG, "config: '%stype' is not a string", w.c_str());
+        if (type->str == "mlstm") {
+            L.mixer = MLSTM;
+            L.heads = rd.integer(*mx, "heads", wm); L.dim = rd.integer(*mx, "dim", wm); L.vdim = rd.integer(*mx, "vdim", wm); L.kv_heads = L.heads;
+            L.gate_cap = rd.num(*mx, "gate_cap", wm);
+            if (rd.err.empty() && !(L.gate_cap > 0)) return fail(NVR_ERR_INVALID_ARG, "config: '%sgate_cap' must be positive", wm.c_str());
+        } else if (type->str == "parallel") {
+            L.mixer = ATTN_GRU;
+            const Json *lf = rd.need(*mx, "left", wm), *rt = rd.need(*mx, "right", wm);
+            if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+            const std::string wl = wm + "left.";
+            L.heads = rd.integer(*lf, "heads", wl); L.kv_heads = rd.integer(*lf, "kv_heads", wl); L.dim = rd.integer(*lf, "dim", wl); L.vdim = rd.integer(*lf, "vdim", wl);
+            L.scale = rd.num(*lf, "scale", wl);
+            if (const Json *m = rd.need(*lf, "mask", wl)) L.window = rd.integer(*m, "size", wl + "mask.");
+            if (const Json *t = rd.need(*lf, "q_temp", wl)) { L.temp_coef = rd.num(*t, "coef", wl + "q_temp."); L.temp_every = rd.integer(*t, "every", wl + "q_temp."); }
+            L.gru_width = rd.integer(*rt, "width", wm + "right.");
+            if (rd.err.empty() && (L.window < 1 || L.temp_every < 1 || L.gru_width < 1))
+                return fail(NVR_ERR_INVALID_ARG, "config: %s mask.size, q_temp.every and right.width must be positive", wm.c_str());
+        } else return fail(NVR_ERR_UNSUPPORTED, "config: layer type '%s' (mlstm or parallel)", type->str.c_str());
+        const Json *mlp = lj.get("mlp");
+        if (mlp && !mlp->is_null()) {
+            const Json *kind = rd.need(*mlp, "kind", w + "mlp.");
+            if (kind && !(kind->kind == Json::Str && kind->str == "dense")) return fail(NVR_ERR_UNSUPPORTED, "config: '%smlp.kind' (dense)", w.c_str());
+            L.has_mlp = true; L.ff_kind = FF_RELU2; L.ff = rd.integer(*mlp, "ff", w + "mlp.");
+            if (rd.err.empty() && L.ff < 1) return fail(NVR_ERR_INVALID_ARG, "config: '%smlp.ff' must be positive", w.c_str());
+        }
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (L.heads < 1 || L.dim < 1 || L.vdim < 1 || L.kv_heads < 1 || L.heads % L.kv_heads)
+            return fail(NVR_ERR_INVALID_ARG, "config: %s %ld heads over %ld key/value heads of %ld / %ld", w.c_str(), (long)L.heads, (long)L.kv_heads, (long)L.dim, (long)L.vdim);
+        const Json *wof = lj.get("weights_of");
+        if (wof && !wof->is_null()) {
+            int64_t j = rd.integer(lj, "weights_of", w);
+            if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+            if (j < 0 || j >= (int64_t)i) return fail(NVR_ERR_INVALID_ARG, "config: '%sweights_of' must name an earlier layer", w.c_str());
+            if (s->layers[(size_t)j].weights_of >= 0) j = s->layers[(size_t)j].weights_of;          // (a borrower's source)
+            const Layer &o = s->layers[(size_t)j];
+            if (o.mixer != L.mixer || o.heads != L.heads || o.kv_heads != L.kv_heads || o.dim != L.dim || o.vdim != L.vdim || o.gru_width != L.gru_width || o.has_mlp != L.has_mlp || o.ff != L.ff)
+                return fail(NVR_ERR_INVALID_ARG, "config: '%sweights_of' names a layer of other sizes", w.c_str());
+            L.weights_of = j;
+        }
+        s->layers.push_back(L); s->runs.push_back((int)(L.weights_of >= 0 ? L.weights_of : (int64_t)i));
     }
     return NVR_OK;
 }
