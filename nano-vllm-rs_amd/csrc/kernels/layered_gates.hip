@@ -54,26 +54,42 @@ __global__ __launch_bounds__(256) void embed_pos_kernel(const ET *__restrict__ E
 }
 
 // ------------------------------------------------------------------------------------------------ exponential gates of a matrix memory
-// One thread per (sequence, head) walks the sequence's rows in order: the running maximum is a scalar recurrence.
-__global__ __launch_bounds__(64) void exp_gates_kernel(const float *__restrict__ pre, int64_t ldp, const float *__restrict__ bi, const float *__restrict__ bfg, float cap, Batch b, int H,
-                                                       float *__restrict__ mstate, float *__restrict__ tok_gate, float *__restrict__ floor_out) {
-    const int sq = blockIdx.x, h = blockIdx.y * 64 + threadIdx.x;
-    if (h >= H) return;
+// One workgroup per (sequence, head), 256 rows at a time: every thread computes the two log gates of its row, one thread walks the running maximum through the
+// 256 rows (an addition and a maximum per row: the only part that is a recurrence), every thread then takes its row's exponentials.  The arithmetic per row is that
+// of a walk row by row, so the result does not depend on where a prompt is cut.
+__global__ __launch_bounds__(256) void exp_gates_kernel(const float *__restrict__ pre, int64_t ldp, const float *__restrict__ bi, const float *__restrict__ bfg, float cap, Batch b, int H,
+                                                        float *__restrict__ mstate, float *__restrict__ tok_gate, float *__restrict__ floor_out) {
+    __shared__ float gis[256], gfs[256], ms[257];
+    const int sq = blockIdx.x, h = blockIdx.y;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0;
-    float *ms = mstate + (int64_t)b.slot[sq] * H + h;
-    float m = b.start[sq] > 0 ? *ms : 0.f;
+    float *mst = mstate + (int64_t)b.slot[sq] * H + h;
+    if (threadIdx.x == 0) ms[0] = b.start[sq] > 0 ? *mst : 0.f;
     const float vbi = bi[h], vbf = bfg[h], icap = 1.0f / cap;
-    for (int i = 0; i < n; ++i) {
-        const int64_t t = r0 + i;
-        const float gi = cap * tanhf((pre[t * ldp + h] + vbi) * icap);
-        const float gf = log_sigmoid_f(cap * tanhf((pre[t * ldp + H + h] + vbf) * icap));
-        const float mn = fmaxf(gf + m, gi);
-        tok_gate[(t * H + h) * 2] = expf(gf + m - mn);
-        tok_gate[(t * H + h) * 2 + 1] = expf(gi - mn);
-        floor_out[t * H + h] = expf(-mn);
-        m = mn;
+    for (int i0 = 0; i0 < n; i0 += 256) {
+        const int nb = min(256, n - i0), i = threadIdx.x;
+        const int64_t t = r0 + i0 + i;
+        float gi = 0.f, gf = 0.f;
+        if (i < nb) {
+            gi = cap * tanhf((pre[t * ldp + h] + vbi) * icap);
+            gf = log_sigmoid_f(cap * tanhf((pre[t * ldp + H + h] + vbf) * icap));
+            gis[i] = gi; gfs[i] = gf;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float m = ms[0];
+            for (int k = 0; k < nb; ++k) { m = fmaxf(gfs[k] + m, gis[k]); ms[k + 1] = m; }
+        }
+        __syncthreads();
+        if (i < nb) {
+            const float mp = ms[i], mn = ms[i + 1];
+            tok_gate[(t * H + h) * 2] = expf(gf + mp - mn);
+            tok_gate[(t * H + h) * 2 + 1] = expf(gi - mn);
+            floor_out[t * H + h] = expf(-mn);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) ms[0] = ms[nb];
     }
-    *ms = m;
+    if (threadIdx.x == 0) *mst = ms[0];       // (thread 0 wrote it last)
 }
 
 // one wave per (row, head)
@@ -227,7 +243,7 @@ int exp_gates(const float *pre, int64_t ldp, const float *bi, const float *bf, f
               hipStream_t s) {
     if (b.T == 0) return 0;
     if (!(cap > 0.f)) return nvr::fail(NVR_ERR_INVALID_ARG, "exp_gates: the gates' cap must be positive");
-    exp_gates_kernel<<<dim3((unsigned)b.B, (unsigned)((H + 63) / 64)), dim3(64), 0, s>>>(pre, ldp, bi, bf, cap, b, (int)H, mstate, tok_gate, floor_out);
+    exp_gates_kernel<<<dim3((unsigned)b.B, (unsigned)H), dim3(256), 0, s>>>(pre, ldp, bi, bf, cap, b, (int)H, mstate, tok_gate, floor_out);
     return launched("exp_gates");
 }
 

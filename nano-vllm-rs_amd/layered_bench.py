@@ -1,4 +1,4 @@
-"""Prefill and decode throughput of the layer-list designs (Rugudra, Pusunex) beside the dense Qwen3 graph at equal sizes (bench.py --layered-compare).
+"""Prefill and decode throughput of the layer-list designs (Rugudra, Pusunex, Sosutar) beside the dense Qwen3 graph at equal sizes (bench.py --layered-compare).
 
 Random weights, layer shapes that resemble a real model's; both models go through the same engine (scheduler, block manager, runner step).
 Per size one JSON object: tokens/s of one prefill step over BATCH prompts of PROMPT tokens and of the decode steps that follow, for both."""
@@ -123,6 +123,58 @@ def pusunex_weights(cfg, seed=0):
     return out
 
 
+def sosutar_config(s, window=512):
+    """Layers in turn: a matrix memory without a feed-forward, then windowed attention beside a gated recurrence of the model's width with a dense feed-forward;
+    from the third layer on a matrix-memory layer uses the first one's weights (a state of its own)."""
+    H, G, D, W = s["heads"], s["kv_heads"], s["dim"], s["width"]
+    layers = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            L = {"type": "mlstm", "mixer": {"heads": H, "dim": D, "vdim": D, "gate_cap": 15.0}, "mlp": None}
+            if i >= 2:
+                L["weights_of"] = 0
+        else:
+            L = {"type": "parallel", "mixer": {"left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "mask": {"size": window}, "q_temp": {"coef": 0.2, "every": 256}, "scale": D ** -0.5},
+                                               "right": {"width": W}}, "mlp": {"kind": "dense", "ff": s["ff"]}}
+        layers.append(L)
+    return {"architecture": "Sosutar", "vocab": s["vocab"], "width": W, "max_positions": 4096, "embedding": {"scale": 4.0}, "logit_scale": 0.5, "norm": {"eps": 1e-5}, "layers": layers}
+
+
+def sosutar_weights(cfg, seed=0):
+    rng = np.random.default_rng(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def lin(o, i, g=1.0):
+        return (rng.standard_normal((o, i), dtype=np.float32) * (g / np.sqrt(i))).astype(np.float32)
+
+    def gains(n, mean=1.0):
+        return (mean + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    out = {"embed": rng.standard_normal((V, W), dtype=np.float32), "pos": rng.standard_normal((cfg["max_positions"], W), dtype=np.float32), "head": lin(V, W), "final.norm": gains(W)}
+    for i, L in enumerate(cfg["layers"]):
+        if L.get("weights_of") is not None:
+            continue
+        m, p = L["mixer"], "l%d." % i
+        out[p + "norm1"], out[p + "ls1"] = gains(W), gains(W, 0.5)
+        if L["type"] == "mlstm":
+            H, D, Dv = m["heads"], m["dim"], m["vdim"]
+            out[p + "mix.q"], out[p + "mix.k"], out[p + "mix.v"], out[p + "mix.g"], out[p + "mix.o"] = lin(H * D, W), lin(H * D, W), lin(H * Dv, W), lin(H * Dv, W), lin(W, H * Dv)
+            out[p + "mix.norm"], out[p + "mix.i"], out[p + "mix.f"] = gains(H * Dv), lin(H, W), lin(H, W)
+            out[p + "mix.i.b"], out[p + "mix.f.b"] = rng.standard_normal(H).astype(np.float32), (3.0 + rng.standard_normal(H)).astype(np.float32)
+        else:
+            a, g = m["left"], m["right"]["width"]
+            H, G, D, Dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            q = p + "mix.left."
+            out[q + "q"], out[q + "k"], out[q + "v"], out[q + "g"], out[q + "o"] = lin(H * D, W), lin(G * D, W), lin(G * Dv, W), lin(H * Dv, W), lin(W, H * Dv)
+            out[q + "q.norm"], out[q + "k.norm"], out[q + "sink"], out[q + "out"] = gains(H * D), gains(G * D), rng.standard_normal(H).astype(np.float32), gains(W)
+            q = p + "mix.right."
+            out[q + "z"], out[q + "x"], out[q + "g"], out[q + "o"] = lin(g, W), lin(g, W), lin(g, W), lin(W, g)
+            out[q + "z.b"], out[q + "x.b"], out[q + "out"] = rng.standard_normal(g).astype(np.float32), (0.5 * rng.standard_normal(g)).astype(np.float32), gains(W)
+        if L.get("mlp"):
+            F = L["mlp"]["ff"]
+            out[p + "norm2"], out[p + "ls2"], out[p + "mlp.up"], out[p + "mlp.down"] = gains(W), gains(W, 0.5), lin(F, W), lin(W, F)
+    return out
+
+
 def _run(nvr, engine, vocab, batch, prompt, steps, warmup):
     sp = nvr.SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True)
     for i in range(batch):
@@ -168,6 +220,14 @@ def compare(nvr, sizes=("w1024", "w2048"), batch=16, prompt=1024, steps=32, warm
                 eng.model_runner.load_tensor(k, np.asarray(v))
             _run(nvr, eng, s["vocab"], 2, 64, 2, 1)
             line["pusunex"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
+            del eng
+        if "sosutar" in which:
+            cfg = sosutar_config(s)
+            eng = nvr.LLMEngine(nvr.Config(**ecfg), nvr.ModelSpec(cfg))
+            for k, v in sosutar_weights(cfg).items():
+                eng.model_runner.load_tensor(k, np.asarray(v))
+            _run(nvr, eng, s["vocab"], 2, 64, 2, 1)
+            line["sosutar"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
             del eng
         if "qwen3" in which:
             m = nvr.ModelConfig(vocab_size=s["vocab"], hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
