@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void exp_gates_kernel(const float *__restrict_
     if (threadIdx.x == 0) *mst = ms[0];       // (thread 0 wrote it last)
 }
 
-// one wave per (row, head)
+// one wave per (row, head); heads of up to 256 values are read once and kept in registers
 template <class OT>
 __global__ __launch_bounds__(256) void memory_readout_kernel(const float *__restrict__ o, const float *__restrict__ floor_in, const OT *__restrict__ gate, int64_t ldg, int64_t gcol, int H,
                                                              int Dv, float eps, const float *__restrict__ w, OT *__restrict__ out, int64_t ldo) {
@@ -102,6 +102,24 @@ __global__ __launch_bounds__(256) void memory_readout_kernel(const float *__rest
     const float *r = o + (t * H + h) * (int64_t)(Dv + 1);
     const float inv_den = 1.0f / (fmaxf(fabsf(r[Dv]), floor_in[t * H + h]) + 1e-6f);
     float ss = 0.f;
+    if (Dv <= 256) {
+        float v[4], gt[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int c = lane + 64 * k;
+            v[k] = c < Dv ? r[c] * inv_den : 0.f;
+            gt[k] = c < Dv ? ld_f(gate, t * ldg + gcol + (int64_t)h * Dv + c) : 0.f;
+            ss += v[k] * v[k];
+        }
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int c = lane + 64 * k;
+            const int64_t col = (int64_t)h * Dv + c;
+            if (c < Dv) st_f(out, t * ldo + col, v[k] * inv * w[col] * sigmoid_f(gt[k]));
+        }
+        return;
+    }
     for (int c = lane; c < Dv; c += 64) { const float v = r[c] * inv_den; ss += v * v; }
     const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
     for (int c = lane; c < Dv; c += 64) {
@@ -154,36 +172,129 @@ __global__ __launch_bounds__(256) void qkv_norm_store_kernel(QkvNormArgs a, Batc
     }
 }
 
+// The same for 16-bit rows whose parts all start and end at multiples of 8 numbers: 16-byte loads and stores, the two sums of squares in one reduction.
+__global__ __launch_bounds__(256) void qkv_norm_store8_kernel(QkvNormArgs a, Batch b) {
+    __shared__ float red[8];
+    const int t = blockIdx.x, sq = b.row_seq[t];
+    const int p = b.start[sq] + (t - b.cu[sq]);
+    const int blk = b.block_tables[(int64_t)sq * b.max_blocks + p / b.block_size], jj = p % b.block_size;
+    const int64_t row = (int64_t)blk * b.block_size + jj;
+    bf16_t *pr = (bf16_t *)a.proj + (int64_t)t * a.ld;
+    const int qn = a.H * a.D, kn = a.G * a.D, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float sq2 = 0.f, sk2 = 0.f;
+    for (int c = threadIdx.x * 8; c < qn; c += 2048) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(pr + a.qcol + c); const bf16_t *e = reinterpret_cast<const bf16_t *>(&v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { const float f = ld_f(e, k); sq2 += f * f; }
+    }
+    for (int c = threadIdx.x * 8; c < kn; c += 2048) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(pr + a.kcol + c); const bf16_t *e = reinterpret_cast<const bf16_t *>(&v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { const float f = ld_f(e, k); sk2 += f * f; }
+    }
+    sq2 = wave_sum(sq2); sk2 = wave_sum(sk2);
+    if (lane == 0) { red[wave] = sq2; red[4 + wave] = sk2; }
+    __syncthreads();
+    float fq = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)qn + a.eps);
+    const float fk = 1.0f / sqrtf(((red[4] + red[5]) + (red[6] + red[7])) / (float)kn + a.eps);
+    if (a.temp_every > 0) fq *= 1.0f + a.temp_coef * logf((float)((p + 1) / a.temp_every) + 1.0f);
+    for (int c = threadIdx.x * 8; c < qn; c += 2048) {
+        uint4 v = *reinterpret_cast<const uint4 *>(pr + a.qcol + c); bf16_t *e = reinterpret_cast<bf16_t *>(&v);
+        const float4 w0 = *reinterpret_cast<const float4 *>(a.wq + c), w1 = *reinterpret_cast<const float4 *>(a.wq + c + 4);
+        const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) st_f(e, k, ld_f(e, k) * fq * w[k]);
+        *reinterpret_cast<uint4 *>(pr + a.qcol + c) = v;
+    }
+    bf16_t *kd = (bf16_t *)a.kc + row * kn;
+    for (int c = threadIdx.x * 8; c < kn; c += 2048) {
+        uint4 v = *reinterpret_cast<const uint4 *>(pr + a.kcol + c); bf16_t *e = reinterpret_cast<bf16_t *>(&v);
+        const float4 w0 = *reinterpret_cast<const float4 *>(a.wk + c), w1 = *reinterpret_cast<const float4 *>(a.wk + c + 4);
+        const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) st_f(e, k, ld_f(e, k) * fk * w[k]);
+        *reinterpret_cast<uint4 *>(kd + c) = v;
+    }
+    // values: 16 lanes of 8 numbers per key/value head and pass (heads of up to 128 numbers in one pass), four heads per wave at a time
+    const int Dv = a.Dv, sub = lane >> 4, l16 = lane & 15;
+    bf16_t *vc = (bf16_t *)a.vc;
+    const int64_t grp = ((int64_t)blk * (b.block_size >> 3) + (jj >> 3)) * a.G * Dv;
+    for (int g = wave * 4 + sub; g < (a.G + 15) / 16 * 16; g += 16) {           // (every lane of a wave takes part in the shuffles)
+        const bool on = g < a.G;
+        float ss = 0.f;
+        if (on)
+            for (int c = l16 * 8; c < Dv; c += 128) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(pr + a.vcol + g * Dv + c); const bf16_t *e = reinterpret_cast<const bf16_t *>(&v);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) { const float f = ld_f(e, k); ss += f * f; }
+            }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float f = a.v_unit ? 1.0f / sqrtf(ss / (float)Dv + a.eps) : 1.f;
+        if (on)
+            for (int c = l16 * 8; c < Dv; c += 128) {
+                uint4 v = *reinterpret_cast<const uint4 *>(pr + a.vcol + g * Dv + c); bf16_t *e = reinterpret_cast<bf16_t *>(&v);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) st_f(e, k, ld_f(e, k) * f);
+                if (a.v_grouped) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) vc[(grp + g * Dv + c + k) * 8 + (jj & 7)] = e[k];
+                } else *reinterpret_cast<uint4 *>(vc + (row * a.G + g) * Dv + c) = v;
+            }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ elementwise gated recurrence
-// One thread per (sequence, channel); the rows of a sequence in order, eight at a time in flight (the loads do not depend on the recurrence).
+// A workgroup owns 32 channels of one sequence and walks its rows in tiles of 128.  Per tile: all 256 threads turn the projections of the tile's rows into the
+// recurrence's coefficients a = 1 - z, b = z cand and the output gate silu(g) (the exponentials do not depend on the state) and leave them in LDS; one
+// thread per channel then walks the 128 rows, S <- a S + b, one fused multiply-add per row, leaving S in a's place; all threads write S silu(g).  The walk
+// is row by row whatever the portion, so the result does not depend on where a prompt is cut.  FAST (16-bit operands): exponentials and reciprocals on the
+// hardware's base-2 units, f32 throughout.
+template <bool FAST> __device__ __forceinline__ float sigm(float z) { return FAST ? __frcp_rn(1.0f + __expf(-z)) : 1.0f / (1.0f + expf(-z)); }
+
 template <class CT>
 __global__ __launch_bounds__(256) void gated_unit_kernel(const CT *__restrict__ proj, int64_t ld, int64_t zcol, int64_t ucol, int64_t gcol, const float *__restrict__ bz,
                                                          const float *__restrict__ bu, Batch b, int N, float *__restrict__ state, CT *__restrict__ out, int64_t ldo) {
-    const int sq = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= N) return;
+    constexpr int CH = 32, R = 128, RG = 256 / CH;
+    constexpr bool FAST = sizeof(CT) == 2;
+    __shared__ float A[R * CH], Bc[R * CH], Gs[R * CH];
+    const int sq = blockIdx.y, l = threadIdx.x & (CH - 1), rg = threadIdx.x / CH, c = blockIdx.x * CH + l;
+    const bool live = c < N;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0;
     float *sp = state + (int64_t)b.slot[sq] * N + c;
-    float S = b.start[sq] > 0 ? *sp : 0.f;
-    const float vbz = bz[c], vbu = bu[c];
-    constexpr int U = 8;
-    for (int i0 = 0; i0 < n; i0 += U) {
-        float z[U], u[U], g[U];
-#pragma unroll
-        for (int k = 0; k < U; ++k) {
-            const int64_t t = r0 + min(i0 + k, n - 1);
-            z[k] = ld_f(proj, t * ld + zcol + c); u[k] = ld_f(proj, t * ld + ucol + c); g[k] = ld_f(proj, t * ld + gcol + c);
-        }
-#pragma unroll
-        for (int k = 0; k < U; ++k) {
-            if (i0 + k < n) {
-                const float zz = sigmoid_f(z[k] + vbz), uu = u[k] + vbu;
-                const float cand = uu >= 0.f ? uu + 0.5f : sigmoid_f(uu);
-                S = (1.0f - zz) * S + zz * cand;
-                st_f(out, (int64_t)(r0 + i0 + k) * ldo + c, S * (g[k] * sigmoid_f(g[k])));
+    float S = (live && rg == 0 && b.start[sq] > 0) ? *sp : 0.f;
+    const float vbz = live ? bz[c] : 0.f, vbu = live ? bu[c] : 0.f;
+    for (int i0 = 0; i0 < n; i0 += R) {
+        const int nb = min(R, n - i0);
+        if (live) {
+#pragma unroll 4
+            for (int r = rg; r < nb; r += RG) {
+                const CT *pr = proj + (int64_t)(r0 + i0 + r) * ld + c;
+                const float gg = ld_f(pr, gcol), zz = sigm<FAST>(ld_f(pr, zcol) + vbz), uu = ld_f(pr, ucol) + vbu;
+                const float cand = uu >= 0.f ? uu + 0.5f : sigm<FAST>(uu);
+                A[r * CH + l] = 1.0f - zz; Bc[r * CH + l] = zz * cand; Gs[r * CH + l] = gg * sigm<FAST>(gg);
             }
         }
+        __syncthreads();
+        if (rg == 0 && live) {
+            for (int r = 0; r < nb; r += 8) {                // eight rows' coefficients into registers, eight steps, eight stores (rows past nb are read, never used)
+                float ca[8], cb[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) { ca[k] = A[(r + k) * CH + l]; cb[k] = Bc[(r + k) * CH + l]; }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) if (r + k < nb) { S = ca[k] * S + cb[k]; ca[k] = S; }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) if (r + k < nb) A[(r + k) * CH + l] = ca[k];
+            }
+        }
+        __syncthreads();
+        if (live) {
+#pragma unroll 4
+            for (int r = rg; r < nb; r += RG) st_f(out, (int64_t)(r0 + i0 + r) * ldo + c, A[r * CH + l] * Gs[r * CH + l]);
+        }
+        __syncthreads();
     }
-    *sp = S;
+    if (rg == 0 && live) *sp = S;
 }
 
 // ------------------------------------------------------------------------------------------------ residual joins
@@ -225,6 +336,18 @@ __global__ __launch_bounds__(256) void relu_squared_kernel(const CT *__restrict_
     st_f(out, t * ldo + c, v * v);
 }
 
+// 16-bit rows, 8 numbers per thread (F and both strides multiples of 8, 16-byte aligned rows)
+__global__ __launch_bounds__(256) void relu_squared8_kernel(const bf16_t *__restrict__ z, int64_t ldz, int64_t T, int64_t F8, bf16_t *__restrict__ out, int64_t ldo) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= T * F8) return;
+    const int64_t t = i / F8, c = (i - t * F8) * 8;
+    uint4 v = *reinterpret_cast<const uint4 *>(z + t * ldz + c);
+    bf16_t *e = reinterpret_cast<bf16_t *>(&v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { const float r = fmaxf(ld_f(e, k), 0.f); st_f(e, k, r * r); }
+    *reinterpret_cast<uint4 *>(out + t * ldo + c) = v;
+}
+
 __global__ __launch_bounds__(256) void scale_f32_kernel(float *__restrict__ y, int64_t n, float c) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) y[i] *= c;
@@ -259,7 +382,10 @@ int memory_readout(const float *o, const float *floor_in, const void *gate, int6
 int qkv_norm_store(const QkvNormArgs &a, const Batch &b, bool bf16, hipStream_t s) {
     if (b.T == 0) return 0;
     if (a.v_grouped && b.block_size % 8) return nvr::fail(NVR_ERR_INVALID_ARG, "qkv_norm_store: grouped value pages need pages of a multiple of 8 tokens");
-    if (bf16) qkv_norm_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
+    const bool vec = bf16 && a.wq && a.wk && a.D % 8 == 0 && a.Dv % 8 == 0 && a.ld % 8 == 0 && ((a.qcol | a.kcol | a.vcol) & 7) == 0 &&
+                     (((uintptr_t)a.proj | (uintptr_t)a.kc | (uintptr_t)a.vc | (uintptr_t)a.wq | (uintptr_t)a.wk) & 15) == 0;
+    if (vec) qkv_norm_store8_kernel<<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
+    else if (bf16) qkv_norm_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
     else qkv_norm_store_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
     return launched("qkv_norm_store");
 }
@@ -267,7 +393,7 @@ int qkv_norm_store(const QkvNormArgs &a, const Batch &b, bool bf16, hipStream_t 
 int gated_unit(const void *proj, int64_t ld, int64_t zcol, int64_t ucol, int64_t gcol, const float *bz, const float *bu, const Batch &b, int64_t N, float *state, void *out, int64_t ldo,
                bool bf16, hipStream_t s) {
     if (b.T == 0 || N == 0) return 0;
-    const dim3 grid((unsigned)((N + 255) / 256), (unsigned)b.B);
+    const dim3 grid((unsigned)((N + 31) / 32), (unsigned)b.B);
     if (bf16) gated_unit_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)proj, ld, zcol, ucol, gcol, bz, bu, b, (int)N, state, (bf16_t *)out, ldo);
     else gated_unit_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)proj, ld, zcol, ucol, gcol, bz, bu, b, (int)N, state, (float *)out, ldo);
     return launched("gated_unit");
@@ -284,6 +410,10 @@ int residual_join(const JoinArgs &a, bool bf16, hipStream_t s) {
 
 int relu_squared(const void *z, int64_t ldz, int64_t T, int64_t F, void *out, int64_t ldo, bool bf16, hipStream_t s) {
     if (T * F == 0) return 0;
+    if (bf16 && F % 8 == 0 && ldz % 8 == 0 && ldo % 8 == 0 && (((uintptr_t)z | (uintptr_t)out) & 15) == 0) {
+        relu_squared8_kernel<<<dim3((unsigned)((T * (F / 8) + 255) / 256)), dim3(256), 0, s>>>((const bf16_t *)z, ldz, T, F / 8, (bf16_t *)out, ldo);
+        return launched("relu_squared");
+    }
     const dim3 grid((unsigned)((T * F + 255) / 256));
     if (bf16) relu_squared_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)z, ldz, T, F, (bf16_t *)out, ldo);
     else relu_squared_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)z, ldz, T, F, (float *)out, ldo);
