@@ -553,11 +553,19 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
     const bool tok = !GATED && a.tok_gate != nullptr;
     const float dec = (GATED || tok) ? 0.f : a.decay[h];
     const int Dr = Dv - a.v_ones;
+    // One column of ones (the gated running sum n of the keys) is not given a column block of its own: the launch covers the Dr columns that proj holds, and the
+    // first block also walks n, one row per thread (row part * RMAX + cl of the threads with cl < RMAX), and sums n . q over the threads by shuffles.
+    const bool fold = tok && a.v_ones == 1;
+    const int Dc = fold ? Dr : Dv;                         // columns the launch's blocks cover
     float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
-    const bool live = c < Dv;
+    const bool live = c < Dc;
     float s[RMAX];
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) { const int d = part * RMAX + r; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; }
+    const int dn = part * RMAX + cl;
+    const bool nblock = fold && blockIdx.z == 0, nown = nblock && cl < RMAX && dn < D;
+    float sn = (nown && st > 0) ? S[(int64_t)dn * Dv + Dv - 1] : 0.f;
+    float *partial_n = as + 2 * TB;                        // [TB][8]
     for (int i0 = 0; i0 < n; i0 += TB) {
         const int nb = min(TB, n - i0);
         __syncthreads();
@@ -639,7 +647,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
         }
         for (int idx = threadIdx.x; idx < nb * 32; idx += 256) {
             const int i = idx >> 5, cc = cb + (idx & 31);
-            vs[idx] = cc < Dv ? (cc < Dr ? ld_f((const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld, a.vcol + (int64_t)h * Dr + cc) : 1.f) : 0.f;
+            vs[idx] = cc < Dc ? (cc < Dr ? ld_f((const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld, a.vcol + (int64_t)h * Dr + cc) : 1.f) : 0.f;
         }
         __syncthreads();
         for (int i = 0; i < nb; ++i) {
@@ -680,6 +688,13 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                     if (part * RMAX + r < D) { s[r] = dd * s[r] + kr[r] * v; o += s[r] * qr[r]; }
             }
             partial[(i * 8 + part) * 32 + cl] = o;
+            if (nblock) {                                   // (uniform over the workgroup)
+                float on = 0.f;
+                if (nown) { sn = as[i] * sn + ks[i * D + dn]; on = sn * qs[i * D + dn]; }
+#pragma unroll
+                for (int off = 16; off > 0; off >>= 1) on += __shfl_xor(on, off, 64);      // over the 32 lanes of the part
+                if (cl == 0) partial_n[i * 8 + part] = on;
+            }
         }
         __syncthreads();
         for (int idx = threadIdx.x; idx < nb * 32; idx += 256) {
@@ -687,12 +702,19 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
             float tot = 0.f;
 #pragma unroll
             for (int p2 = 0; p2 < 8; ++p2) tot += partial[(i * 8 + p2) * 32 + (idx & 31)];
-            if (cc < Dv) a.o[(int64_t)(r0 + i0 + i) * a.H * Dv + (int64_t)h * Dv + cc] = tot;
+            if (cc < Dc) a.o[(int64_t)(r0 + i0 + i) * a.H * Dv + (int64_t)h * Dv + cc] = tot;
+        }
+        if (nblock && threadIdx.x < nb) {
+            float tot = 0.f;
+#pragma unroll
+            for (int p2 = 0; p2 < 8; ++p2) tot += partial_n[threadIdx.x * 8 + p2];
+            a.o[(int64_t)(r0 + i0 + threadIdx.x) * a.H * Dv + (int64_t)h * Dv + Dv - 1] = tot;
         }
     }
     if (live)
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) { const int d = part * RMAX + r; if (d < D) S[(int64_t)d * Dv + c] = s[r]; }
+    if (nown) S[(int64_t)dn * Dv + Dv - 1] = sn;
 }
 
 template <class OT>
@@ -902,8 +924,9 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
         else if (bf16) retention_seq_kernel<R_, bf16_t, false><<<grid, dim3(256), 0, s>>>(a, b);     \
         else retention_seq_kernel<R_, float, false><<<grid, dim3(256), 0, s>>>(a, b);                \
     } while (0)
-    const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32 + 32) * 4;
+    const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32 + 32 + 128) * 4;
     if (a.D <= 256 && lds <= 64 * 1024) {                 // (beyond: the token-by-token form, whose LDS does not grow with the key size)
+        const dim3 grid((unsigned)b.B, (unsigned)a.H, (unsigned)(((a.tok_gate && a.v_ones == 1 ? a.Dv - 1 : a.Dv) + 31) / 32));   // (a single column of ones rides in the first block)
 #define NVR_RETB(R_)                                                                                 \
     do {                                                                                             \
         if (gated) { if (bf16) retention_block_kernel<R_, bf16_t, true><<<grid, dim3(256), lds, s>>>(a, b);   \

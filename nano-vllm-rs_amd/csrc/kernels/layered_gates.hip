@@ -100,17 +100,18 @@ __global__ __launch_bounds__(256) void memory_readout_kernel(const float *__rest
     const int h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (h >= H) return;
     const float *r = o + (t * H + h) * (int64_t)(Dv + 1);
-    const float inv_den = 1.0f / (fmaxf(fabsf(r[Dv]), floor_in[t * H + h]) + 1e-6f);
     float ss = 0.f;
     if (Dv <= 256) {
         float v[4], gt[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < 4; ++k) {                   // (every load of the wave goes out before the first is used)
             const int c = lane + 64 * k;
-            v[k] = c < Dv ? r[c] * inv_den : 0.f;
+            v[k] = c < Dv ? r[c] : 0.f;
             gt[k] = c < Dv ? ld_f(gate, t * ldg + gcol + (int64_t)h * Dv + c) : 0.f;
-            ss += v[k] * v[k];
         }
+        const float inv_den = 1.0f / (fmaxf(fabsf(r[Dv]), floor_in[t * H + h]) + 1e-6f);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { v[k] *= inv_den; ss += v[k] * v[k]; }
         const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -120,6 +121,7 @@ __global__ __launch_bounds__(256) void memory_readout_kernel(const float *__rest
         }
         return;
     }
+    const float inv_den = 1.0f / (fmaxf(fabsf(r[Dv]), floor_in[t * H + h]) + 1e-6f);
     for (int c = lane; c < Dv; c += 64) { const float v = r[c] * inv_den; ss += v * v; }
     const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
     for (int c = lane; c < Dv; c += 64) {
@@ -264,16 +266,31 @@ __global__ __launch_bounds__(256) void gated_unit_kernel(const CT *__restrict__ 
     float *sp = state + (int64_t)b.slot[sq] * N + c;
     float S = (live && rg == 0 && b.start[sq] > 0) ? *sp : 0.f;
     const float vbz = live ? bz[c] : 0.f, vbu = live ? bu[c] : 0.f;
+    // the projections of a tile's rows are requested one tile ahead, into registers: they arrive while the tile before is walked and written
+    CT zr[R / RG], ur[R / RG], gr[R / RG];
+    auto request = [&](int i0) {
+        const int nb = min(R, n - i0);
+#pragma unroll
+        for (int k = 0; k < R / RG; ++k) {
+            const int r = min(rg + k * RG, nb - 1);
+            const CT *pr = proj + (int64_t)(r0 + i0 + r) * ld + c;
+            zr[k] = pr[zcol]; ur[k] = pr[ucol]; gr[k] = pr[gcol];
+        }
+    };
+    if (live && n > 0) request(0);
     for (int i0 = 0; i0 < n; i0 += R) {
         const int nb = min(R, n - i0);
         if (live) {
-#pragma unroll 4
-            for (int r = rg; r < nb; r += RG) {
-                const CT *pr = proj + (int64_t)(r0 + i0 + r) * ld + c;
-                const float gg = ld_f(pr, gcol), zz = sigm<FAST>(ld_f(pr, zcol) + vbz), uu = ld_f(pr, ucol) + vbu;
-                const float cand = uu >= 0.f ? uu + 0.5f : sigm<FAST>(uu);
-                A[r * CH + l] = 1.0f - zz; Bc[r * CH + l] = zz * cand; Gs[r * CH + l] = gg * sigm<FAST>(gg);
+#pragma unroll
+            for (int k = 0; k < R / RG; ++k) {
+                const int r = rg + k * RG;
+                if (r < nb) {
+                    const float gg = ld_f(&gr[k], 0), zz = sigm<FAST>(ld_f(&zr[k], 0) + vbz), uu = ld_f(&ur[k], 0) + vbu;
+                    const float cand = uu >= 0.f ? uu + 0.5f : sigm<FAST>(uu);
+                    A[r * CH + l] = 1.0f - zz; Bc[r * CH + l] = zz * cand; Gs[r * CH + l] = gg * sigm<FAST>(gg);
+                }
             }
+            if (i0 + R < n) request(i0 + R);
         }
         __syncthreads();
         if (rg == 0 && live) {
