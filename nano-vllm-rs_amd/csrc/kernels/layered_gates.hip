@@ -252,7 +252,9 @@ __global__ __launch_bounds__(256) void qkv_norm_store8_kernel(QkvNormArgs a, Bat
 // thread per channel then walks the 128 rows, S <- a S + b, one fused multiply-add per row, leaving S in a's place; all threads write S silu(g).  The walk
 // is row by row whatever the portion, so the result does not depend on where a prompt is cut.  FAST (16-bit operands): exponentials and reciprocals on the
 // hardware's base-2 units, f32 throughout.
-template <bool FAST> __device__ __forceinline__ float sigm(float z) { return FAST ? __frcp_rn(1.0f + __expf(-z)) : 1.0f / (1.0f + expf(-z)); }
+template <bool FAST> __device__ __forceinline__ float sigm(float z) {
+    return FAST ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z)) : 1.0f / (1.0f + expf(-z));       // (2^+inf = inf, 1 / inf = 0: no overflow on the way)
+}
 
 template <class CT>
 __global__ __launch_bounds__(256) void gated_unit_kernel(const CT *__restrict__ proj, int64_t ld, int64_t zcol, int64_t ucol, int64_t gcol, const float *__restrict__ bz,
@@ -260,7 +262,10 @@ __global__ __launch_bounds__(256) void gated_unit_kernel(const CT *__restrict__ 
     constexpr int CH = 32, R = 128, RG = 256 / CH;
     constexpr bool FAST = sizeof(CT) == 2;
     __shared__ float A[R * CH], Bc[R * CH], Gs[R * CH];
-    const int sq = blockIdx.y, l = threadIdx.x & (CH - 1), rg = threadIdx.x / CH, c = blockIdx.x * CH + l;
+    // consecutive workgroups go to the 8 XCDs in turn: with a grid of a multiple of 8 channel groups, XCD x takes the groups x * (groups / 8) ..., so that the
+    // 64-byte pieces of one 128-byte line of a row meet in one L2
+    const int ngrp = gridDim.x, bx = (ngrp & 7) == 0 ? (int)(blockIdx.x & 7) * (ngrp >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const int sq = blockIdx.y, l = threadIdx.x & (CH - 1), rg = threadIdx.x / CH, c = bx * CH + l;
     const bool live = c < N;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0;
     float *sp = state + (int64_t)b.slot[sq] * N + c;

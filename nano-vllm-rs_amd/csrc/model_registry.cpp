@@ -265,16 +265,29 @@ int LayeredSpec::parse_sosutar(const Json &c, LayeredSpec *s) {
             return fail(NVR_ERR_INVALID_ARG, "config: %s %ld heads over %ld key/value heads of %ld / %ld", w.c_str(), (long)L.heads, (long)L.kv_heads, (long)L.dim, (long)L.vdim);
         const Json *wof = lj.get("weights_of");
         if (wof && !wof->is_null()) {
-            int64_t j = rd.integer(lj, "weights_of", w);
+            L.weights_of = rd.integer(lj, "weights_of", w);
             if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
-            if (j < 0 || j >= (int64_t)i) return fail(NVR_ERR_INVALID_ARG, "config: '%sweights_of' must name an earlier layer", w.c_str());
-            if (s->layers[(size_t)j].weights_of >= 0) j = s->layers[(size_t)j].weights_of;          // (a borrower's source)
-            const Layer &o = s->layers[(size_t)j];
-            if (o.mixer != L.mixer || o.heads != L.heads || o.kv_heads != L.kv_heads || o.dim != L.dim || o.vdim != L.vdim || o.gru_width != L.gru_width || o.has_mlp != L.has_mlp || o.ff != L.ff)
-                return fail(NVR_ERR_INVALID_ARG, "config: '%sweights_of' names a layer of other sizes", w.c_str());
-            L.weights_of = j;
         }
-        s->layers.push_back(L); s->runs.push_back((int)(L.weights_of >= 0 ? L.weights_of : (int64_t)i));
+        s->layers.push_back(L);
+    }
+    // a layer may name any other layer (also a later one, or one that borrows itself): the tensors are those of the layer the chain ends at
+    const int64_t n = (int64_t)s->layers.size();
+    std::vector<int64_t> src((size_t)n);
+    for (int64_t i = 0; i < n; ++i) {
+        int64_t j = i, hops = 0;
+        while (s->layers[(size_t)j].weights_of >= 0 || s->layers[(size_t)j].weights_of < -1) {
+            const int64_t k = s->layers[(size_t)j].weights_of;
+            if (k < 0 || k >= n || k == j || ++hops > n) return fail(NVR_ERR_INVALID_ARG, "config: 'layers[%ld].weights_of' must name another layer that leads to tensors", (long)i);
+            j = k;
+        }
+        src[(size_t)i] = j;
+        const Layer &o = s->layers[(size_t)j], &L = s->layers[(size_t)i];
+        if (o.mixer != L.mixer || o.heads != L.heads || o.kv_heads != L.kv_heads || o.dim != L.dim || o.vdim != L.vdim || o.gru_width != L.gru_width || o.has_mlp != L.has_mlp || o.ff != L.ff)
+            return fail(NVR_ERR_INVALID_ARG, "config: 'layers[%ld].weights_of' names a layer of other sizes", (long)i);
+    }
+    for (int64_t i = 0; i < n; ++i) {
+        if (src[(size_t)i] != i) s->layers[(size_t)i].weights_of = src[(size_t)i];
+        s->runs.push_back((int)src[(size_t)i]);
     }
     return NVR_OK;
 }

@@ -8,7 +8,7 @@ name -> array with the checkpoint's tensor names.  Linear weights are [out, in].
   layer:     x <- x + ls1 * mixer(n1(x));   x <- x + ls2 * ff(n2(x))   (a layer without a feed-forward has the first half only)
   n(v)    =  w * v / sqrt(mean(v^2) + eps)
   logits  =  head n_final(x) * logit_scale
-A layer with 'weights_of': j reads layer j's tensors and keeps a state / cache of its own.
+A layer with 'weights_of': j reads layer j's tensors (j may come later) and keeps a state / cache of its own.
 """
 import math
 
@@ -143,8 +143,10 @@ def forward(cfg, wt, tokens, layer_outputs=None, pos0=0, states=None):
     x = wt["embed"][tokens] * cfg["embedding"]["scale"] + wt["pos"][pos0 + np.arange(T)]
     new_states = []
     for i, L in enumerate(cfg["layers"]):
-        src = L.get("weights_of", i)
-        p = "l%d." % (i if src is None else src)
+        src = i
+        while cfg["layers"][src].get("weights_of") is not None:     # (a borrowed layer may borrow itself)
+            src = cfg["layers"][src]["weights_of"]
+        p = "l%d." % src
         st = states[i] if states is not None else None
         h = rms(x, eps) * wt[p + "norm1"]
         if L["type"] == "mlstm":

@@ -38,6 +38,7 @@ MECHANISMS = {
     "attention_keys_of_32_values_of_48": make_config([side_layer(heads=8, kv_heads=1, dim=32, vdim=48, window=24, gru=16)]),
     "attention_twenty_heads_on_one": make_config([side_layer(heads=20, kv_heads=1, dim=32, vdim=16, window=9, gru=16)]),
     "shared_weights": make_config([mlstm_layer(), side_layer(), mlstm_layer(weights_of=0), side_layer(weights_of=1), mlstm_layer(weights_of=0)]),
+    "shared_weights_named_ahead": make_config([mlstm_layer(weights_of=2), side_layer(ff=None), mlstm_layer(), side_layer(ff=None, weights_of=1), mlstm_layer(weights_of=0)]),
     "scales_of_one": make_config([side_layer(), mlstm_layer(ff=24)], embedding_scale=1.0, logit_scale=1.0),
 }
 

@@ -20,6 +20,11 @@ def test_registry_reads_the_design():
     assert "Sosutar" in nvr.registered_architectures()
     s = nvr.ModelSpec(small())
     assert (s.architecture, s.family, s.vocab_size, s.num_layer_runs) == ("Sosutar", 1, 53, 6)
+    cfg = small()                                                  # a layer may name a later one, or one that borrows itself
+    cfg["layers"][0], cfg["layers"][3] = cfg["layers"][3], cfg["layers"][0]
+    cfg["layers"][0]["weights_of"] = 3
+    cfg["layers"].append(dict(cfg["layers"][0], weights_of=0))
+    assert nvr.ModelSpec(cfg).num_layer_runs == 7
 
 
 @pytest.mark.parametrize("breakage, message", [
@@ -33,7 +38,9 @@ def test_registry_reads_the_design():
     (lambda c: c["layers"][1]["mixer"]["left"].update(kv_heads=3), "4 heads over 3 key/value heads"),
     (lambda c: c["layers"][1]["mixer"].pop("right"), "mixer.right' is missing"),
     (lambda c: c["layers"][1]["mlp"].update(kind="moe"), "mlp.kind"),
-    (lambda c: c["layers"][3].update(weights_of=3), "must name an earlier layer"),
+    (lambda c: c["layers"][3].update(weights_of=3), "must name another layer"),
+    (lambda c: c["layers"][3].update(weights_of=9), "must name another layer"),
+    (lambda c: (c["layers"][0].update(weights_of=3), c["layers"][3].update(weights_of=0)), "must name another layer"),
     (lambda c: c["layers"][3].update(weights_of=1), "layer of other sizes"),
     (lambda c: c["layers"][4]["mixer"]["right"].update(width=8), "layer of other sizes"),
 ])
