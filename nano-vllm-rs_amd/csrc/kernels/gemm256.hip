@@ -32,7 +32,8 @@
 
 namespace nvr { namespace NVR_DT_NS {
 
-enum { GEPI_F16 = 0, GEPI_RESID = 1, GEPI_SILU = 2, GEPI_ROPE = 3, GEPI_LMHEAD = 4 };   // RESID: y is the residual stream: y <- fp16(y + fp16(x·Wᵀ)) (qwen3.rs:382,389)
+enum { GEPI_F16 = 0, GEPI_RESID = 1, GEPI_SILU = 2, GEPI_ROPE = 3, GEPI_LMHEAD = 4, GEPI_RELU2 = 5 };   // RELU2: y = max(x·Wᵀ, 0)² (the product rounded to 16 bits first, as the unfused pair of launches does)
+//   // RESID: y is the residual stream: y <- fp16(y + fp16(x·Wᵀ)) (qwen3.rs:382,389)
 // LMHEAD (r06): the LM head over >= 128 rows (ParallelLMHead::compute_logits, embed_head.rs:292-306, + the greedy branch of Sampler::forward,
 // sampler.rs:109-112): W = the [V, hidden] head, nothing is written as fp16 — every tile leaves (max, lowest vocabulary index) of its 256
 // columns per token row (pval / pidx [column tile][T], merged by argmax_partials) and, on demand, the f32 logits straight from the accumulators;
@@ -359,7 +360,11 @@ __global__ __launch_bounds__(512) void gemm256_kernel(const half_t *__restrict__
                     for (int b = 0; b < 2; ++b)
 #pragma unroll
                         for (int j = 0; j < 2; ++j) {
-                            const float4_t v = acc[a][i][b][j];
+                            float4_t v = acc[a][i][b][j];
+                            if (EPI == GEPI_RELU2) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) { const float r = fmaxf((float)(half_t)v[e], 0.f); v[e] = r * r; }
+                            }
                             pk[a][i][b][j] = (half4_t){(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
                         }
         }
@@ -380,7 +385,7 @@ __global__ __launch_bounds__(512) void gemm256_kernel(const half_t *__restrict__
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int ml = wm * 32 + j * 16 + r;                      // token row inside the half
-                if (EPI == GEPI_F16 || EPI == GEPI_RESID || EPI == GEPI_ROPE) {
+                if (EPI == GEPI_F16 || EPI == GEPI_RESID || EPI == GEPI_ROPE || EPI == GEPI_RELU2) {
 #pragma unroll
                     for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -496,7 +501,8 @@ static int g256_prepare() {                                               // 128
     const void *fns[] = {reinterpret_cast<const void *>(&gemm256_kernel<GEPI_F16>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_SILU>),
                          reinterpret_cast<const void *>(&gemm256_kernel<GEPI_ROPE, 128>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_ROPE, 64>),
                          reinterpret_cast<const void *>(&gemm256_kernel<GEPI_RESID>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_LMHEAD>),
-                         reinterpret_cast<const void *>(&gemm256_kernel<GEPI_F16, 0, true>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_SILU, 0, true>)};
+                         reinterpret_cast<const void *>(&gemm256_kernel<GEPI_F16, 0, true>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_SILU, 0, true>),
+                         reinterpret_cast<const void *>(&gemm256_kernel<GEPI_RELU2>)};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * G_BUF + 4096);
         if (e != hipSuccess) return nvr::fail(NVR_ERR_HIP, "gemm256: hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -537,6 +543,15 @@ int gemm256(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int6
     gemm256_kernel<GEPI_F16><<<dim3((unsigned)g256_grid(tt)), dim3(512), 2 * G_BUF, s>>>((const half_t *)x, ldx, (const half_t *)W, (int)T, (int)K,
                                                                                         (int)N, (int)N, (half_t *)y, G256Epi{}, tx, tt / tx, g256_cg(tx, tt / tx, false));
     return g256_check("gemm256");
+}
+// y = max(x . W^T, 0)^2: a dense feed-forward's up product with its squared ReLU in the epilogue
+int gemm256_relu2(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int64_t K, int64_t N, half_bits *y, hipStream_t s) {
+    if (!gemm256_ok(T, K, N, ldx)) return nvr::fail(NVR_ERR_UNSUPPORTED, "gemm256_relu2: T=%ld K=%ld N=%ld", (long)T, (long)K, (long)N);
+    if (int rc = g256_prepare()) return rc;
+    const int tx = (int)(N / 256), tt = tx * (int)((T + 255) / 256);
+    gemm256_kernel<GEPI_RELU2><<<dim3((unsigned)g256_grid(tt)), dim3(512), 2 * G_BUF, s>>>((const half_t *)x, ldx, (const half_t *)W, (int)T, (int)K,
+                                                                                          (int)N, (int)N, (half_t *)y, G256Epi{}, tx, tt / tx, g256_cg(tx, tt / tx, false));
+    return g256_check("gemm256_relu2");
 }
 // Rows grouped by expert (a mixture of experts over many tokens): T is a multiple of 256 and row block rb multiplies the matrix W + row_w[rb] * w_stride
 // (row_w on the device: the host does not know how many rows an expert got).  y = x . W_e^T, or out = silu(gate) * up with W_e = [gate rows; up rows].

@@ -109,6 +109,7 @@ bool gemm256_ok(int64_t T, int64_t K, int64_t N, int64_t ldx);
 bool gemm256_silu_ok(int64_t T, int64_t K, int64_t I, int64_t ldx);
 bool gemm256_rope_ok(int64_t T, int64_t K, int64_t H, int64_t KVH, int64_t D, int64_t ldx);
 int gemm256(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int64_t K, int64_t N, half_bits *y, hipStream_t s);
+int gemm256_relu2(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int64_t K, int64_t N, half_bits *y, hipStream_t s);   // y = max(x . W^T, 0)^2
 int gemm256_grouped(const half_bits *x, int64_t ldx, const half_bits *W, int64_t w_stride, const int32_t *row_w, int64_t T, int64_t K, int64_t N, half_bits *y, hipStream_t s);
 int gemm256_grouped_silu_mul(const half_bits *x, int64_t ldx, const half_bits *W, int64_t w_stride, const int32_t *row_w, int64_t T, int64_t K, int64_t I, half_bits *out, hipStream_t s);
 int gemm256_resid(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int64_t K, int64_t N, half_bits *h, hipStream_t s);

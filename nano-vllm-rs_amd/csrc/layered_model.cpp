@@ -1044,8 +1044,11 @@ int LayeredModel::forward_scaled(nvr_model_runner &r, const StepPlan &p) {
         }
         RC(kl::residual_join(j, bf16, s));
         if (L.has_mlp) {
-            RC(gemm(r, a2, W, w.up, T, W, L.ff, gu));
-            RC(kl::relu_squared(gu, L.ff, T, L.ff, act, L.ff, bf16, s));
+            if (bf16 && nvr::kb::gemm256_preferred(T, W, L.ff, W)) RC(nvr::kb::gemm256_relu2((const uint16_t *)a2, W, (const uint16_t *)w.up, T, W, L.ff, (uint16_t *)act, s));   // (the squared ReLU in the product's epilogue)
+            else {
+                RC(gemm(r, a2, W, w.up, T, W, L.ff, gu));
+                RC(kl::relu_squared(gu, L.ff, T, L.ff, act, L.ff, bf16, s));
+            }
             RC(gemm(r, act, L.ff, w.down, T, L.ff, W, tmp));
             kl::JoinArgs j2{}; j2.x = x; j2.T = T; j2.W = W; j2.eps = eps; j2.ls = w.ls2; j2.y1 = tmp; j2.ld1 = W; j2.wn = next_n1; j2.out = a1; j2.ldo = W;
             RC(kl::residual_join(j2, bf16, s));

@@ -222,6 +222,18 @@ def test_long_prompts_and_decoding_with_split_keys(dtype):
     check(np.concatenate(ga)[:40], wa[:40], dtype, "first rows")
 
 
+def test_squared_relu_in_the_products_epilogue():
+    """A step of more than four thousand rows at a width of 1024: the feed-forward's first product takes the 256 x 256 tiles with the squared ReLU in its epilogue; the same
+    prompt in two portions takes the product and the activation as two launches.  Both must agree with the restatement."""
+    cfg = make_config([mlstm_layer(heads=1, dim=16, vdim=16, ff=2048)], vocab=47, width=1024, max_positions=4400)
+    w = make_weights(cfg, seed=29, pos_gain=0.5)
+    toks = tokens_of(4300, cfg["vocab"], 30)
+    want = expected_logits(cfg, w, toks)
+    for cuts in ([4300], [2100, 2200]):
+        got = Driver(cfg, w, "bfloat16", page=64, pages=70, slots=1, max_tokens=4352, max_len=4400).run_alone(toks, cuts=cuts)
+        check(got[::7], want[::7], "bfloat16", f"portions {cuts}")
+
+
 def test_decode_steps_replay_a_graph():
     """Decode-sized steps are captured the second time their shape is seen and replayed from then on; every replay is compared."""
     cfg = everything(); w = make_weights(cfg, seed=16)
