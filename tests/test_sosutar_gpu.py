@@ -27,6 +27,7 @@ MECHANISMS = {
     "matrix_memory_one_head_small_cap": make_config([mlstm_layer(heads=1, dim=40, vdim=8, gate_cap=1.5)]),
     "matrix_memory_values_of_31_and_32": make_config([mlstm_layer(heads=3, dim=8, vdim=31), mlstm_layer(heads=2, dim=24, vdim=32)]),
     "matrix_memory_keys_of_128": make_config([mlstm_layer(heads=1, dim=128, vdim=16, gate_cap=20.0)]),
+    "matrix_memory_heads_of_64_and_128": make_config([mlstm_layer(heads=2, dim=64, vdim=96), mlstm_layer(heads=1, dim=128, vdim=136, gate_cap=6.0)], width=96),
     "matrix_memory_with_feed_forward": make_config([mlstm_layer(ff=40)]),
     "attention_beside_recurrence": make_config([side_layer(heads=4, kv_heads=2, dim=16, vdim=16, window=12, gru=40)]),
     "attention_one_head_window_of_one": make_config([side_layer(heads=1, kv_heads=1, dim=24, vdim=8, window=1, gru=8, ff=None)]),
