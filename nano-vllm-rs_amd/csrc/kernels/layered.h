@@ -53,6 +53,10 @@ struct SinkAttnArgs {
     const float *slope;                      // a linear distance penalty instead of the logarithmic one: score -= slope[h] * (i - j) (null: none; not together with r1 / r2).
                                              // The tiled form takes it as its table (linear_penalty_table)
     int32_t window;                          // > 0: position i sees only the keys j with i - j < window (itself and the window - 1 before it); 0: every key j <= i
+    int32_t chunk;                           // > 0: position i sees only the keys j <= i of its own chunk, floor(j / chunk) == floor(i / chunk), chunks counted from position 0
+    float softcap;                           // > 0: score <- softcap * tanh(score / softcap) (after the scale, before any bias)
+    const float *gate_bias;                  // not null: no softmax — the weight of a visible key is sigmoid(score + gate_bias[h]), not normalised over the keys
+                                             // (general form and gate_attention_tiled; not together with a penalty or a sink)
 };
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);     // any shape; a context that fits the LDS score buffer
 // The same on the matrix cores (bf16 operands, D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16).  tiles (device, built by the host): tile i covers the
@@ -82,12 +86,18 @@ struct RetentionArgs {
     // (instead of decay[h]); q is scaled by qscale.  v_ones: the last v_ones of the Dv value columns are not read from proj (whose value rows hold Dv - v_ones
     // numbers per head): their value is 1 for every token, so that the state's column is the gated running sum of the keys and o's column its product with q.
     const float *tok_gate; int32_t v_ones;
+    // qk_share > 1: that many consecutive heads read the same q and k (head h those of group h / qk_share; proj holds H / qk_share of each): a state-space layer's
+    // input and output maps B and C shared by a group of heads
+    int32_t qk_share;
+    // gated form, decay_exp: the decay is exp(-exp(az + abias)) instead of a power of the sigmoid.  bonus (gated form, [H][D] f32): the output is read BEFORE the update
+    // and sees the current token through the bonus alone, o = (S_(t-1) + diag(bonus_h) k v^T)^T q, then S_t = diag(decay) S_(t-1) + k v^T
+    bool decay_exp; const float *bonus;
 };
 int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s);
 // out[t][h*Dv + c] = o[t][h][c] / rms(o[t][h][:]) * w[c] * silu(gate[t][h*Dv + c]); gate: rows of the operand type (stride ldg) from column gcol; w (one weight per
-// value column, shared by the heads) may be null
+// value column, shared by the heads) may be null; w_heads: w holds a weight per head and column ([H * Dv])
 int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, const float *w, void *out, int64_t ldo,
-                   bool bf16, hipStream_t s);
+                   bool bf16, hipStream_t s, bool w_heads = false);
 
 // g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha * g) * (u + 1); gu: rows [T][2*F] of the operand type (gate columns, then up columns)
 int clamped_glu(const void *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s);
@@ -148,11 +158,15 @@ int silu_mul(const void *gu, int64_t T, int64_t F, void *out, int64_t ldo, bool 
 // grouped by expert: off [E + 1], order [T top] (place -> token * top + choice), place_of (its inverse).  With pad > 1 every expert's rows start at a multiple of pad
 // (places then run up to (T top / pad + E) pad) and row_w[block] names the expert of each of the nblocks blocks of pad rows: the form a tiled product over whole
 // row blocks wants, with the rows brought together by moe_gather (xs[place] = h[token] * score).
+// softmax: score is the chosen experts' share of the softmax over ALL experts, divided by the sum of the chosen shares (+ 1e-20), instead of the sigmoid.
+// extra > 0: rows E .. E + extra - 1 of wr are further f32 projections of h that leave as they are in extra_out[t * extra + i] (a shared expert's gate).
 int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr, int64_t E, int64_t top, int32_t *sel, float *score, int32_t *off, int32_t *order,
-              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s);
+              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s, bool softmax = false, int64_t extra = 0, float *extra_out = nullptr);
 int moe_gather(const void *h, int64_t ldh, int64_t T, int64_t W, int64_t top, const int32_t *place_of, const float *score, void *xs, bool bf16, hipStream_t s);
-// out[t] = sum_k y[place_of[t * top + k]] + shared[t] (shared may be null)
-int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s);
+// out[t] = sum_k y[place_of[t * top + k]] + shared[t] (shared may be null).  With score ([T][top] f32) choice k is weighted by score[t * top + k]; with shared_gate
+// ([T] f32, stride gate_ld) the shared row is multiplied by sigmoid(shared_gate[t * gate_ld]).
+int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s,
+                const float *score = nullptr, const float *shared_gate = nullptr, int64_t gate_ld = 1);
 
 // The per-layer token input is y = Wp (gelu_tanh(Wg x) * E[id][ecol .. ecol + dim)), x += y / rms(y) * wn: two ordinary products with this between them
 // (z = Wg x rows of dim numbers -> g), and its last step inside layer_tail.
@@ -204,12 +218,56 @@ int gated_unit(const void *proj, int64_t ld, int64_t zcol, int64_t ucol, int64_t
 
 // A sublayer's result joins the stream: x[t][c] += ls[c] * r, r = y1 (y2 null) or (y1 / rms(y1) * w1 + y2 / rms(y2) * w2) / 2 (two branches, each normed over the row);
 // with wn also out[t] = x[t] / rms(x[t]) * wn in the operand type (the next sublayer's input).  y rows of the operand type, strides ld1 / ld2; ls may be null (ones).
-struct JoinArgs { float *x; int64_t T, W; float eps; const float *ls; const void *y1; int64_t ld1; const float *w1; const void *y2; int64_t ld2; const float *w2; const float *wn; void *out; int64_t ldo; };
+// add (rows of the operand type, stride lda; may be null) is a further addend that joins as it is: x += ls * r + add (a feed-forward that read the same input as the mixer).
+struct JoinArgs { float *x; int64_t T, W; float eps; const float *ls; const void *y1; int64_t ld1; const float *w1; const void *y2; int64_t ld2; const float *w2; const float *wn; void *out; int64_t ldo;
+                  const void *add; int64_t lda; };
 int residual_join(const JoinArgs &a, bool bf16, hipStream_t s);
 
 // out = max(z, 0)^2 (rows of F numbers, strides ldz / ldo)
 int relu_squared(const void *z, int64_t ldz, int64_t T, int64_t F, void *out, int64_t ldo, bool bf16, hipStream_t s);
 // y[i] *= c (f32, n numbers)
 int scale_f32(float *y, int64_t n, float c, hipStream_t s);
+
+// ---------------------------------------------------------------------------------------------------------------------------------------------------
+// Blocks of layers whose two sublayers read ONE norm, with a token shift in front of the mixer (layered_ssm.hip): a state-space mixer (causal convolution, step
+// sizes, gated group norm; its recurrence is retention's token-gated form with shared input / output maps), rotated keys on their way into the pages, an
+// attention without softmax over chunks of positions, the mixes of a time-mixing recurrence (retention's gated form with a bonus), the input of a pass over a
+// looped range of layers.
+
+// h = x / sqrt(mean(x^2) + eps) * w -> out_h (may be null); m_t = h_t + (h_(t-1) - h_t) * shift -> out_m (operand type; h_(-1) = 0; the row before a chunk comes from
+// hist[par][slot], the chunk's last h goes to hist[par ^ 1][slot]).  hist: [2][slots][W] f32.
+int norm_shift(const float *x, const Batch &b, int64_t W, float eps, const float *w, const float *shift, void *out_h, void *out_m, float *hist, int64_t slots, bool bf16, hipStream_t s);
+
+// out[t] = [x[t] | x0[t]] in the operand type (rows of 2 W numbers): the input of the product that starts a pass over a looped range of layers
+int pair_rows(const float *x, const float *x0, int64_t T, int64_t W, void *out, bool bf16, hipStream_t s);
+
+// The front of a state-space mixer.  In row t of proj (operand type, stride ld) the C channels from column ccol pass a causal convolution per channel over `taps`
+// rows (w: [C][taps] f32, the last column is the current row's; bias [C]) and silu -> out (operand type, stride ldo); rows before position 0 are zero, the taps - 1 rows
+// before a chunk come from hist[par][slot] ([2][slots][taps - 1][C] f32) and the chunk's last taps - 1 inputs go to the other half.  The H step sizes at column dcol:
+// dt = softplus(z + dt_bias[h]); tok_gate[(t * H + h) * 2] = (exp(-exp(a_log[h]) * dt), dt): retention's token-gated form takes them.
+struct ConvGateArgs { const void *proj; int64_t ld, ccol, dcol; int32_t C, taps, H; const float *w, *bias, *dt_bias, *a_log; float *hist; int64_t slots; void *out; int64_t ldo; float *tok_gate; };
+int conv_gates(const ConvGateArgs &a, const Batch &b, bool bf16, hipStream_t s);
+
+// The end of a state-space mixer: y[t][h][c] = o[t][h][c] + skip[h] * xs[t][h * Dv + c] (o f32 [T][H * Dv], xs rows of the operand type, stride ldx); y *= silu(z) (z rows,
+// stride ldz); y is RMS-normed in `groups` equal consecutive parts of the H * Dv numbers, times w -> out (operand type, stride ldo).
+struct StateReadoutArgs { const float *o; const void *xs; int64_t ldx; const void *z; int64_t ldz; const float *skip, *w; int32_t T, H, Dv, groups; float eps; void *out; int64_t ldo; };
+int state_readout(const StateReadoutArgs &a, bool bf16, hipStream_t s);
+
+// Rotated queries and keys ('rotate half': coordinate i < rot / 2 of a head pairs with i + rot / 2, angle = position * freq[i], f32) for an attention over pages: q rotated in
+// place in proj, k rotated -> the K page row of the position, v -> the V page row (layouts as kv_store).  freq: [rot / 2] f32 on the device.
+struct RopeStoreArgs { void *proj; int64_t ld, qcol, kcol, vcol; int32_t H, G, D, Dv, rot; const float *freq; void *kc, *vc; bool v_grouped; };
+int rope_store(const RopeStoreArgs &a, const Batch &b, bool bf16, hipStream_t s);
+
+// out[t][i * W ...] = m_t + (m_(t-1) - m_t) * mu[i] for i < n (mu: [n][W] f32; m rows of the operand type, stride ldm; m_(-1) = 0; history as norm_shift, hist [2][slots][W] f32
+// of m): the inputs of a time-mixing layer's projections, side by side in rows of n W numbers
+int shift_mixes(const void *m, int64_t ldm, const Batch &b, int64_t W, int32_t n, const float *mu, void *out, float *hist, int64_t slots, bool bf16, hipStream_t s);
+
+// y = tanh(y) in place (rows of N numbers, stride ld)
+int tanh_rows(void *y, int64_t ld, int64_t T, int64_t N, bool bf16, hipStream_t s);
+
+// Attention without softmax on the matrix cores (bf16 operands; gate_bias set; D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16): the tiles of sink_attention_tiled,
+// P = sigmoid(capped score + bias) on the visible keys of the row's chunk, O = P V summed over the key tiles.
+bool gate_attention_tiled_ok(const SinkAttnArgs &a, bool bf16, int block_size);
+int gate_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, hipStream_t s);
 
 }}  // namespace nvr::kl

@@ -224,7 +224,10 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
     const CT *kc = (const CT *)a.kc; const CT *vc = (const CT *)a.vc;
     const int32_t *bt = b.block_tables + (int64_t)sq * b.max_blocks;
     const float r1 = a.r1 ? a.r1[h] : 0.f, r2 = a.r2 ? a.r2[h] : 0.f, slope = a.slope ? a.slope[h] : 0.f;
-    const int j0 = a.window > 0 ? max(0, ctx - a.window) : 0;      // first visible key; the score buffer holds the keys j0 .. ctx - 1
+    int j0 = a.window > 0 ? max(0, ctx - a.window) : 0;            // first visible key; the score buffer holds the keys j0 .. ctx - 1
+    if (a.chunk > 0) j0 = max(j0, i / a.chunk * a.chunk);          // (chunks count from position 0 of the sequence)
+    const bool gate = a.gate_bias != nullptr;                      // weights sigmoid(score + bias), not normalised
+    const float gb = gate ? a.gate_bias[h] : 0.f;
     sc -= j0;
     float mx = a.sink ? a.sink[h] : -INFINITY;
     for (int j = j0 + threadIdx.x; j < ctx; j += 256) {
@@ -235,15 +238,21 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
         float s = dot * a.scale;
         if (a.r1) s -= r1 * log1pf(r2 * (float)(i - j));
         if (a.slope) s -= slope * (float)(i - j);
+        if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
+        if (gate) s = 1.0f / (1.0f + expf(-(s + gb)));
         sc[j] = s;
         mx = fmaxf(mx, s);
     }
+    float inv = 1.0f;
+    if (gate) __syncthreads();                          // (publishes the weights)
+    else {
     mx = block_max<256>(mx, red);
     float sum = 0.f;
     for (int j = j0 + threadIdx.x; j < ctx; j += 256) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
     sum = block_sum<256>(sum, red);                     // (its barriers also publish the weights)
     if (a.sink) sum += expf(a.sink[h] - mx);
-    const float inv = 1.0f / sum;
+    inv = 1.0f / sum;
+    }
     // values: column c by lanes, keys split over the 256 / CW groups
     float *part = sc + ctx;                             // (behind the last score)
     const int64_t vld = a.vld ? a.vld : a.Dv;           // (values inside the key rows: the latent of latent attention)
@@ -475,27 +484,29 @@ __global__ __launch_bounds__(64) void sink_attn_merge_kernel(SinkAttnArgs a, Bat
 // log(sigmoid(z)) without overflow
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <int RMAX, class PT, bool GATED>
+template <int RMAX, class PT, int MODE>
 __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Batch b) {
+    constexpr bool GATED = MODE != 0, PRE = MODE == 2;      // PRE: the output is read before the update, the current token enters it through the bonus
     __shared__ float qs[2][512], ks[2][512], red[8][32];
     __shared__ float as[GATED ? 2 : 1][GATED ? 512 : 1];
     const int sq = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * 32;
     const int c = cb + (threadIdx.x & 31), part = threadIdx.x >> 5;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0, st = b.start[sq];
     const int D = a.D, Dv = a.Dv, half = a.rot_dims / 2;
+    const int hq = a.qk_share > 1 ? h / a.qk_share : h;    // the head whose q and k this head reads
     const bool tok = !GATED && a.tok_gate != nullptr;     // (keep, take) per token and head instead of decay[h]
     const float dec = (GATED || tok) ? 0.f : a.decay[h];
     const int Dr = Dv - a.v_ones;                          // value columns that proj holds; the rest are ones
     float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
     const bool live = c < Dv;
-    float s[RMAX];
+    float s[RMAX], ub[PRE ? RMAX : 1];
 #pragma unroll
-    for (int r = 0; r < RMAX; ++r) { const int d = part + r * 8; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; }
+    for (int r = 0; r < RMAX; ++r) { const int d = part + r * 8; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; if (PRE) ub[PRE ? r : 0] = d < D ? a.bonus[(int64_t)h * D + d] : 0.f; }
     for (int i = 0; i < n; ++i) {
         const int t = r0 + i, buf = i & 1;
         const float keep = tok ? a.tok_gate[((int64_t)t * a.H + h) * 2] : dec, take = tok ? a.tok_gate[((int64_t)t * a.H + h) * 2 + 1] : 1.f;
         const PT *pr = (const PT *)a.proj + (int64_t)t * a.ld;
-        const PT *q = pr + a.qcol + (int64_t)h * D, *k = pr + a.kcol + (int64_t)h * D;
+        const PT *q = pr + a.qcol + (int64_t)hq * D, *k = pr + a.kcol + (int64_t)hq * D;
         for (int d = threadIdx.x; d < D; d += 256) {
             float qv = ld_f(q, d), kv = ld_f(k, d);
             if (d < a.rot_dims) {
@@ -507,7 +518,8 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
             }
             if (GATED) {
                 qv *= a.qscale;
-                as[buf][d] = expf(log_sigmoid(ld_f((const PT *)a.az, (int64_t)t * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d]) * a.inv_tau);
+                const float z = ld_f((const PT *)a.az, (int64_t)t * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d];
+                as[buf][d] = a.decay_exp ? expf(-expf(z)) : expf(log_sigmoid(z) * a.inv_tau);
             }
             if (tok) { qv *= a.qscale; kv *= take; }
             qs[buf][d] = qv; ks[buf][d] = kv * a.kscale;
@@ -518,7 +530,10 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
             const int d = part + r * 8;
-            if (d < D) { s[r] = (GATED ? as[buf][d] : keep) * s[r] + ks[buf][d] * v; o += s[r] * qs[buf][d]; }
+            if (d < D) {
+                if (PRE) { const float kv = ks[buf][d] * v; o += (s[r] + ub[PRE ? r : 0] * kv) * qs[buf][d]; s[r] = as[buf][d] * s[r] + kv; }
+                else { s[r] = (GATED ? as[buf][d] : keep) * s[r] + ks[buf][d] * v; o += s[r] * qs[buf][d]; }
+            }
         }
         red[part][threadIdx.x & 31] = o;
         __syncthreads();
@@ -540,11 +555,13 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
 // barrier later they are summed over the 8 row groups.  Token order and arithmetic per token are those of the token-by-token kernel: the result does not depend
 // on where a prompt is cut.  Thread (c, part) owns rows part * RMAX .. part * RMAX + RMAX - 1 of column c.
 // GATED: the decay is per token and key channel, sigmoid(z + bias)^(1/tau) with z from rows of the operand type, and q is scaled by qscale (gated linear attention).
-template <int RMAX, class PT, bool GATED>
+template <int RMAX, class PT, int MODE>
 __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, Batch b) {
+    constexpr bool GATED = MODE != 0, PRE = MODE == 2;
     constexpr int TB = 16;
     extern __shared__ float rsm[];
     const int D = a.D, Dv = a.Dv, half = a.rot_dims / 2;
+    const int hq = a.qk_share > 1 ? (int)blockIdx.y / a.qk_share : (int)blockIdx.y;
     float *qs = rsm, *ks = qs + TB * D, *vs = ks + TB * D, *partial = vs + TB * 32;      // [TB][D], [TB][D], [TB][32], [TB][8][32]
     float *as = partial + TB * 8 * 32;                                                    // GATED: [TB][D] decays; token-gated: [TB] keep, [TB] take
     const int sq = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * 32;
@@ -559,9 +576,9 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
     const int Dc = fold ? Dr : Dv;                         // columns the launch's blocks cover
     float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
     const bool live = c < Dc;
-    float s[RMAX];
+    float s[RMAX], ub[PRE ? RMAX : 1];
 #pragma unroll
-    for (int r = 0; r < RMAX; ++r) { const int d = part * RMAX + r; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; }
+    for (int r = 0; r < RMAX; ++r) { const int d = part * RMAX + r; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; if (PRE) ub[PRE ? r : 0] = d < D ? a.bonus[(int64_t)h * D + d] : 0.f; }
     const int dn = part * RMAX + cl;
     const bool nblock = fold && blockIdx.z == 0, nown = nblock && cl < RMAX && dn < D;
     float sn = (nown && st > 0) ? S[(int64_t)dn * Dv + Dv - 1] : 0.f;
@@ -581,7 +598,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
             for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
                 const int i = idx / cpt, d0 = (idx - i * cpt) << 3;
                 const bf16_t *pr = (const bf16_t *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
-                const bf16_t *q = pr + a.qcol + (int64_t)h * D + d0, *k = pr + a.kcol + (int64_t)h * D + d0;
+                const bf16_t *q = pr + a.qcol + (int64_t)hq * D + d0, *k = pr + a.kcol + (int64_t)hq * D + d0;
                 const uint4 ql = *reinterpret_cast<const uint4 *>(q), qh = *reinterpret_cast<const uint4 *>(q + half);
                 const uint4 kl = *reinterpret_cast<const uint4 *>(k), kh = *reinterpret_cast<const uint4 *>(k + half);
                 const int64_t p = st + i0 + i;
@@ -603,14 +620,14 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
             for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
                 const int i = idx / cpt, d0 = (idx - i * cpt) << 3;
                 const bf16_t *pr = (const bf16_t *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
-                const uint4 qv = *reinterpret_cast<const uint4 *>(pr + a.qcol + (int64_t)h * D + d0), kv = *reinterpret_cast<const uint4 *>(pr + a.kcol + (int64_t)h * D + d0);
+                const uint4 qv = *reinterpret_cast<const uint4 *>(pr + a.qcol + (int64_t)hq * D + d0), kv = *reinterpret_cast<const uint4 *>(pr + a.kcol + (int64_t)hq * D + d0);
                 const uint4 zv = *reinterpret_cast<const uint4 *>((const bf16_t *)a.az + (int64_t)(r0 + i0 + i) * a.ldz + (int64_t)h * D + d0);
                 const bf16_t *qe = reinterpret_cast<const bf16_t *>(&qv), *ke = reinterpret_cast<const bf16_t *>(&kv), *ze = reinterpret_cast<const bf16_t *>(&zv);
                 const float *bp = a.abias + (int64_t)h * D + d0;
 #pragma unroll
                 for (int y = 0; y < 8; ++y) {
                     qs[i * D + d0 + y] = ld_f(qe, y) * a.qscale; ks[i * D + d0 + y] = ld_f(ke, y) * a.kscale;
-                    as[i * D + d0 + y] = exp2f(-a.inv_tau * __log2f(1.0f + exp2f(-kLog2e * (ld_f(ze, y) + bp[y]))));
+                    as[i * D + d0 + y] = a.decay_exp ? exp2f(-kLog2e * exp2f(kLog2e * (ld_f(ze, y) + bp[y]))) : exp2f(-a.inv_tau * __log2f(1.0f + exp2f(-kLog2e * (ld_f(ze, y) + bp[y]))));
                 }
             }
         } else if (tok && sizeof(PT) == 2 && a.rot_dims == 0 && (D & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol) & 7) == 0 && ((uintptr_t)a.proj & 15) == 0) {
@@ -619,7 +636,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
             for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
                 const int i = idx / cpt, d0 = (idx - i * cpt) << 3;
                 const bf16_t *pr = (const bf16_t *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
-                const uint4 qv = *reinterpret_cast<const uint4 *>(pr + a.qcol + (int64_t)h * D + d0), kv = *reinterpret_cast<const uint4 *>(pr + a.kcol + (int64_t)h * D + d0);
+                const uint4 qv = *reinterpret_cast<const uint4 *>(pr + a.qcol + (int64_t)hq * D + d0), kv = *reinterpret_cast<const uint4 *>(pr + a.kcol + (int64_t)hq * D + d0);
                 const bf16_t *qe = reinterpret_cast<const bf16_t *>(&qv), *ke = reinterpret_cast<const bf16_t *>(&kv);
                 const float take = as[TB + i];
 #pragma unroll
@@ -629,7 +646,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
         for (int idx = threadIdx.x; idx < nb * D; idx += 256) {
             const int i = dsh >= 0 ? idx >> dsh : idx / D, d = idx - i * D;
             const PT *pr = (const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
-            const PT *q = pr + a.qcol + (int64_t)h * D, *k = pr + a.kcol + (int64_t)h * D;
+            const PT *q = pr + a.qcol + (int64_t)hq * D, *k = pr + a.kcol + (int64_t)hq * D;
             float qv = ld_f(q, d), kv = ld_f(k, d);
             if (d < a.rot_dims) {
                 const int fi = d < half ? d : d - half;
@@ -640,7 +657,8 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
             }
             if (GATED) {
                 qv *= a.qscale;
-                as[idx] = expf(log_sigmoid(ld_f((const PT *)a.az, (int64_t)(r0 + i0 + i) * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d]) * a.inv_tau);
+                const float z = ld_f((const PT *)a.az, (int64_t)(r0 + i0 + i) * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d];
+                as[idx] = a.decay_exp ? expf(-expf(z)) : expf(log_sigmoid(z) * a.inv_tau);
             }
             if (tok) { qv *= a.qscale; kv *= as[TB + i]; }
             qs[idx] = qv; ks[idx] = kv * a.kscale;
@@ -665,11 +683,17 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                         *reinterpret_cast<float4 *>(aa + r) = *reinterpret_cast<const float4 *>(ar + r);
                     }
 #pragma unroll
-                    for (int r = 0; r < RMAX; ++r) { s[r] = aa[r] * s[r] + kk[r] * v; o += s[r] * qq[r]; }
+                    for (int r = 0; r < RMAX; ++r) {
+                        if (PRE) { const float kv = kk[r] * v; o += (s[r] + ub[PRE ? r : 0] * kv) * qq[r]; s[r] = aa[r] * s[r] + kv; }
+                        else { s[r] = aa[r] * s[r] + kk[r] * v; o += s[r] * qq[r]; }
+                    }
                 } else {
 #pragma unroll
                     for (int r = 0; r < RMAX; ++r)
-                        if (part * RMAX + r < D) { s[r] = ar[r] * s[r] + kr[r] * v; o += s[r] * qr[r]; }
+                        if (part * RMAX + r < D) {
+                            if (PRE) { const float kv = kr[r] * v; o += (s[r] + ub[PRE ? r : 0] * kv) * qr[r]; s[r] = ar[r] * s[r] + kv; }
+                            else { s[r] = ar[r] * s[r] + kr[r] * v; o += s[r] * qr[r]; }
+                        }
                 }
             } else if (D == 8 * RMAX) {
                 const float dd = tok ? as[i] : dec;
@@ -719,7 +743,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
 
 template <class OT>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float *__restrict__ o, const OT *__restrict__ gate, int64_t ldg, int64_t gcol, int H, int Dv,
-                                                             float eps, const float *__restrict__ w, OT *__restrict__ out, int64_t ldo) {
+                                                             float eps, const float *__restrict__ w, OT *__restrict__ out, int64_t ldo, int w_heads) {
     const int64_t t = blockIdx.x; const int lane = threadIdx.x & 63;
     for (int h = threadIdx.x >> 6; h < H; h += 4) {              // a wave per head
         const float *orow = o + (t * H + h) * Dv;
@@ -729,7 +753,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float *__rest
         const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
         for (int c = lane; c < Dv; c += 64) {
             const float g = ld_f(gate, t * ldg + gcol + (int64_t)h * Dv + c);
-            st_f(out, t * ldo + (int64_t)h * Dv + c, orow[c] * r * (w ? w[c] : 1.0f) * (g / (1.0f + expf(-g))));
+            st_f(out, t * ldo + (int64_t)h * Dv + c, orow[c] * r * (w ? w[w_heads ? h * Dv + c : c] : 1.0f) * (g / (1.0f + expf(-g))));
         }
     }
 }
@@ -897,7 +921,9 @@ int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t
     if (b.T == 0) return 0;
     if (a.G < 1 || a.H % a.G) return nvr::fail(NVR_ERR_INVALID_ARG, "sink_attention: %d heads over %d key/value heads", a.H, a.G);
     if ((a.r1 || a.r2) && a.slope) return nvr::fail(NVR_ERR_INVALID_ARG, "sink_attention: a logarithmic and a linear penalty together");
-    const size_t keys = a.window > 0 ? (size_t)std::min(b.max_ctx, a.window) : (size_t)b.max_ctx;
+    size_t keys = a.window > 0 ? (size_t)std::min(b.max_ctx, a.window) : (size_t)b.max_ctx;
+    if (a.chunk > 0) keys = std::min(keys, (size_t)a.chunk);
+    if (a.gate_bias && (a.r1 || a.r2 || a.slope || a.sink)) return nvr::fail(NVR_ERR_INVALID_ARG, "sink_attention: gated weights take no penalty and no sink");
     const size_t lds = ((size_t)a.D + keys + 256) * 4;
     if (lds > kMaxLds) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention: %zu visible keys do not fit the score buffer", keys);
     const dim3 grid((unsigned)b.T, (unsigned)a.H);
@@ -915,24 +941,30 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
     const bool gated = a.az != nullptr;
     if (gated && !a.abias) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: gated decays need their bias");
     if (gated && a.tok_gate) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: decays per channel and gates per token together");
+    if (a.bonus && !gated) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: a bonus belongs to the gated form");
+    if (a.qk_share > 1 && a.H % a.qk_share) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: %d heads in groups of %d", a.H, a.qk_share);
     if (a.v_ones < 0 || a.v_ones >= a.Dv) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: %d of %d value columns are ones", a.v_ones, a.Dv);
     if (!gated && !a.tok_gate && !a.decay) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: no decay");
 #define NVR_RET(R_)                                                                                  \
     do {                                                                                             \
-        if (gated) { if (bf16) retention_seq_kernel<R_, bf16_t, true><<<grid, dim3(256), 0, s>>>(a, b);   \
-                     else retention_seq_kernel<R_, float, true><<<grid, dim3(256), 0, s>>>(a, b); }       \
-        else if (bf16) retention_seq_kernel<R_, bf16_t, false><<<grid, dim3(256), 0, s>>>(a, b);     \
-        else retention_seq_kernel<R_, float, false><<<grid, dim3(256), 0, s>>>(a, b);                \
+        if (gated && a.bonus) { if (bf16) retention_seq_kernel<R_, bf16_t, 2><<<grid, dim3(256), 0, s>>>(a, b);   \
+                                else retention_seq_kernel<R_, float, 2><<<grid, dim3(256), 0, s>>>(a, b); }       \
+        else if (gated) { if (bf16) retention_seq_kernel<R_, bf16_t, 1><<<grid, dim3(256), 0, s>>>(a, b);   \
+                     else retention_seq_kernel<R_, float, 1><<<grid, dim3(256), 0, s>>>(a, b); }       \
+        else if (bf16) retention_seq_kernel<R_, bf16_t, 0><<<grid, dim3(256), 0, s>>>(a, b);     \
+        else retention_seq_kernel<R_, float, 0><<<grid, dim3(256), 0, s>>>(a, b);                \
     } while (0)
     const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32 + 32 + 128) * 4;
     if (a.D <= 256 && lds <= 64 * 1024) {                 // (beyond: the token-by-token form, whose LDS does not grow with the key size)
         const dim3 grid((unsigned)b.B, (unsigned)a.H, (unsigned)(((a.tok_gate && a.v_ones == 1 ? a.Dv - 1 : a.Dv) + 31) / 32));   // (a single column of ones rides in the first block)
 #define NVR_RETB(R_)                                                                                 \
     do {                                                                                             \
-        if (gated) { if (bf16) retention_block_kernel<R_, bf16_t, true><<<grid, dim3(256), lds, s>>>(a, b);   \
-                     else retention_block_kernel<R_, float, true><<<grid, dim3(256), lds, s>>>(a, b); }       \
-        else if (bf16) retention_block_kernel<R_, bf16_t, false><<<grid, dim3(256), lds, s>>>(a, b); \
-        else retention_block_kernel<R_, float, false><<<grid, dim3(256), lds, s>>>(a, b);            \
+        if (gated && a.bonus) { if (bf16) retention_block_kernel<R_, bf16_t, 2><<<grid, dim3(256), lds, s>>>(a, b);   \
+                                else retention_block_kernel<R_, float, 2><<<grid, dim3(256), lds, s>>>(a, b); }       \
+        else if (gated) { if (bf16) retention_block_kernel<R_, bf16_t, 1><<<grid, dim3(256), lds, s>>>(a, b);   \
+                     else retention_block_kernel<R_, float, 1><<<grid, dim3(256), lds, s>>>(a, b); }       \
+        else if (bf16) retention_block_kernel<R_, bf16_t, 0><<<grid, dim3(256), lds, s>>>(a, b); \
+        else retention_block_kernel<R_, float, 0><<<grid, dim3(256), lds, s>>>(a, b);            \
     } while (0)
         if (rows <= 8) NVR_RETB(8);
         else if (rows <= 16) NVR_RETB(16);
@@ -949,11 +981,11 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
 }
 
 int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, const float *w, void *out, int64_t ldo,
-                   bool bf16, hipStream_t s) {
+                   bool bf16, hipStream_t s, bool w_heads) {
     if (T == 0) return 0;
     const dim3 grid((unsigned)T);
-    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(o, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (bf16_t *)out, ldo);
-    else head_norm_gate_kernel<float><<<grid, dim3(256), 0, s>>>(o, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (float *)out, ldo);
+    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(o, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (bf16_t *)out, ldo, w_heads ? 1 : 0);
+    else head_norm_gate_kernel<float><<<grid, dim3(256), 0, s>>>(o, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (float *)out, ldo, w_heads ? 1 : 0);
     return launched("head_norm_gate");
 }
 

@@ -508,19 +508,31 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const OT *__restrict__ gu
 
 // ------------------------------------------------------------------------------------------------ mixture of experts
 // Router: z = Wr h in f32; the `top` largest logits of a token (the lower index wins a tie) go to sel, their sigmoid to score ([T][top]).  The logits and not the
-// scores are compared: the order is the same, and saturated scores do not tie.
+// scores are compared: the order is the same, and saturated scores do not tie.  softmax: the score of a chosen expert is its share e^(z - max) / sum over ALL experts,
+// divided by the sum of the chosen shares (+ 1e-20).  Rows E .. E + extra - 1 of wr are further projections of h whose values leave as they are.
 template <class OT>
 __global__ __launch_bounds__(256) void moe_route_kernel(const OT *__restrict__ h, int64_t ldh, int W, const float *__restrict__ wr, int E, int top,
-                                                        int32_t *__restrict__ sel, float *__restrict__ score) {
-    extern __shared__ float sc[];                       // [E]
+                                                        int32_t *__restrict__ sel, float *__restrict__ score, int softmax, int extra, float *__restrict__ extra_out) {
+    extern __shared__ float sc[];                       // [E + extra]
     const int64_t t = blockIdx.x; const int lane = threadIdx.x & 63;
-    for (int e = threadIdx.x >> 6; e < E; e += 4) {
+    for (int e = threadIdx.x >> 6; e < E + extra; e += 4) {
         float d = 0.f;
         for (int c = lane; c < W; c += 64) d = fmaf(ld_f(h, t * ldh + c), wr[(int64_t)e * W + c], d);
         d = wave_sum(d);
-        if (lane == 0) sc[e] = d;
+        if (lane == 0) { sc[e] = d; if (e >= E) extra_out[t * extra + (e - E)] = d; }
     }
     __syncthreads();
+    float zmax = 0.f, zsum = 1.f;
+    if (softmax && threadIdx.x < 64) {                  // (the first wave keeps both for its choices below)
+        zmax = -INFINITY;
+        for (int e = lane; e < E; e += 64) zmax = fmaxf(zmax, sc[e]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) zmax = fmaxf(zmax, __shfl_xor(zmax, o, 64));
+        zsum = 0.f;
+        for (int e = lane; e < E; e += 64) zsum += expf(sc[e] - zmax);
+        zsum = wave_sum(zsum);
+    }
+    float chosen = 0.f;                                 // (lane 0: the sum of the chosen shares)
     for (int k = 0; k < top; ++k) {                     // the first wave: top times the arg-max over the experts' logits
         if (threadIdx.x < 64) {
             float best = -INFINITY; int bi = E;
@@ -531,10 +543,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const OT *__restrict__ h
                 if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
             }
             if (bi >= E) bi = E - 1;                        // (logits that are not numbers compare false everywhere: the index still has to be an expert's)
-            if (lane == 0) { sel[t * top + k] = bi; score[t * top + k] = sigmoid_f(best); sc[bi] = -INFINITY; }
+            if (lane == 0) {
+                const float sv = softmax ? expf(best - zmax) / zsum : sigmoid_f(best);
+                sel[t * top + k] = bi; score[t * top + k] = sv; chosen += sv; sc[bi] = -INFINITY;
+            }
         }
         __syncthreads();
     }
+    if (softmax && threadIdx.x == 0) for (int k = 0; k < top; ++k) score[t * top + k] /= chosen + 1e-20f;
 }
 
 // One workgroup: counts per expert, offsets, and a place for every (token, choice) among its expert's rows.  order[place] = token * top + choice;
@@ -574,11 +590,12 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const OT *__restrict__ 
 // out[t] = sum_k y[place_of[t * top + k]] (+ shared[t]) in the operand type
 template <class OT>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const OT *__restrict__ y, const int32_t *__restrict__ place_of, int top, const OT *__restrict__ shared, int W,
-                                                          OT *__restrict__ out) {
+                                                          OT *__restrict__ out, const float *__restrict__ score, const float *__restrict__ shared_gate, int64_t gate_ld) {
     const int64_t t = blockIdx.x;
+    const float sg = (shared && shared_gate) ? sigmoid_f(shared_gate[t * gate_ld]) : 1.f;
     for (int c = threadIdx.x; c < W; c += 256) {
-        float v = shared ? ld_f(shared, t * W + c) : 0.f;
-        for (int k = 0; k < top; ++k) v += ld_f(y, (int64_t)place_of[t * top + k] * W + c);
+        float v = shared ? ld_f(shared, t * W + c) * sg : 0.f;
+        for (int k = 0; k < top; ++k) v += ld_f(y, (int64_t)place_of[t * top + k] * W + c) * (score ? score[t * top + k] : 1.f);
         st_f(out, t * W + c, v);
     }
 }
@@ -768,12 +785,13 @@ int silu_mul(const void *gu, int64_t T, int64_t F, void *out, int64_t ldo, bool 
 }
 
 int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr, int64_t E, int64_t top, int32_t *sel, float *score, int32_t *off, int32_t *order,
-              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s) {
+              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s, bool softmax, int64_t extra, float *extra_out) {
     if (T == 0) return 0;
+    if (extra < 0 || (extra > 0 && !extra_out)) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: %ld further rows without a place for them", (long)extra);
     if (top < 1 || top > E) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: %ld of %ld experts", (long)top, (long)E);
     if ((size_t)(E + 1) * 4 > 60000) return nvr::fail(NVR_ERR_UNSUPPORTED, "moe_route: %ld experts", (long)E);
-    if (bf16) moe_route_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), (size_t)E * 4, s>>>((const bf16_t *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score);
-    else moe_route_kernel<float><<<dim3((unsigned)T), dim3(256), (size_t)E * 4, s>>>((const float *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score);
+    if (bf16) moe_route_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), (size_t)(E + extra) * 4, s>>>((const bf16_t *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score, softmax ? 1 : 0, (int)extra, extra_out);
+    else moe_route_kernel<float><<<dim3((unsigned)T), dim3(256), (size_t)(E + extra) * 4, s>>>((const float *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score, softmax ? 1 : 0, (int)extra, extra_out);
     if (int rc = launched("moe_route")) return rc;
     if (pad < 1) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: rows padded to %ld", (long)pad);
     moe_group_kernel<<<dim3(1), dim3(1024), (size_t)(E + 1) * 4, s>>>(sel, (int)(T * top), (int)E, (int)pad, (int)nblocks, off, order, place_of, row_w);
@@ -787,10 +805,11 @@ int moe_gather(const void *h, int64_t ldh, int64_t T, int64_t W, int64_t top, co
     return launched("moe_gather");
 }
 
-int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s) {
+int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s,
+                const float *score, const float *shared_gate, int64_t gate_ld) {
     if (T == 0) return 0;
-    if (bf16) moe_combine_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), 0, s>>>((const bf16_t *)y, place_of, (int)top, (const bf16_t *)shared, (int)W, (bf16_t *)out);
-    else moe_combine_kernel<float><<<dim3((unsigned)T), dim3(256), 0, s>>>((const float *)y, place_of, (int)top, (const float *)shared, (int)W, (float *)out);
+    if (bf16) moe_combine_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), 0, s>>>((const bf16_t *)y, place_of, (int)top, (const bf16_t *)shared, (int)W, (bf16_t *)out, score, shared_gate, gate_ld);
+    else moe_combine_kernel<float><<<dim3((unsigned)T), dim3(256), 0, s>>>((const float *)y, place_of, (int)top, (const float *)shared, (int)W, (float *)out, score, shared_gate, gate_ld);
     return launched("moe_combine");
 }
 

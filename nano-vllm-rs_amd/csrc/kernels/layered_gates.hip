@@ -327,7 +327,7 @@ __global__ __launch_bounds__(256) void residual_join_kernel(JoinArgs a) {
     const int64_t t = blockIdx.x;
     const int W = (int)a.W;
     float *xr = a.x + t * W;
-    const YT *y1 = (const YT *)a.y1 + t * a.ld1, *y2 = TWO ? (const YT *)a.y2 + t * a.ld2 : nullptr;
+    const YT *y1 = (const YT *)a.y1 + t * a.ld1, *y2 = TWO ? (const YT *)a.y2 + t * a.ld2 : nullptr, *ad = a.add ? (const YT *)a.add + t * a.lda : nullptr;
     float f1 = 1.f, f2 = 1.f;
     if (TWO) {
         float s1 = 0.f, s2 = 0.f;
@@ -339,7 +339,8 @@ __global__ __launch_bounds__(256) void residual_join_kernel(JoinArgs a) {
     for (int c = threadIdx.x; c < W; c += 256) {
         float r = ld_f(y1, c);
         if (TWO) r = 0.5f * (r * f1 * a.w1[c] + ld_f(y2, c) * f2 * a.w2[c]);
-        const float v = xr[c] + (a.ls ? a.ls[c] * r : r);
+        float v = xr[c] + (a.ls ? a.ls[c] * r : r);
+        if (ad) v += ld_f(ad, c);
         xr[c] = v; sn += v * v;
     }
     if (a.wn) {

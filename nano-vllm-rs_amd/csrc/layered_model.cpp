@@ -49,12 +49,6 @@ LayeredModel::~LayeredModel() {
     for (void *p : owned) if (p) (void)hipFree(p);
 }
 
-template <class T> int LayeredModel::own(T **p, size_t bytes) {            // zeroed device memory that lives as long as the model
-    RC(dmalloc(p, bytes));
-    NVR_HIP_CHECK(hipMemset(*p, 0, bytes ? bytes : 16));
-    owned.push_back((void *)*p);
-    return NVR_OK;
-}
 
 int LayeredModel::init(nvr_model_runner &r) {
     r.env = nvr::Env::read();
@@ -81,6 +75,7 @@ int LayeredModel::init(nvr_model_runner &r) {
 
     if (spec.layout == LayeredSpec::SEQUENTIAL) RC(init_sequential(r));
     else if (spec.layout == LayeredSpec::SCALED) RC(init_scaled(r));
+    else if (spec.layout == LayeredSpec::JOINT) RC(init_joint(r));
     else {
     // weights (zero until loaded)
     const int64_t taps = spec.taps;
@@ -211,6 +206,7 @@ int LayeredModel::load_tensor(nvr_model_runner &r, const char *name_in, int dtyp
     const std::string name(name_in);
     if (spec.layout == LayeredSpec::SEQUENTIAL) return load_sequential(r, name, dtype, shape, ndim, data);
     if (spec.layout == LayeredSpec::SCALED) return load_scaled(r, name, dtype, shape, ndim, data);
+    if (spec.layout == LayeredSpec::JOINT) return load_joint(r, name, dtype, shape, ndim, data);
     const int64_t W = spec.width, V = spec.vocab;
     auto is2 = [&](int64_t a, int64_t b) { return ndim == 2 && shape[0] == a && shape[1] == b; };
     auto bad = [&]() { return fail(NVR_ERR_LEN_MISMATCH, "load_tensor: '%s' has the wrong shape", name_in); };
@@ -395,6 +391,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
 int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
     if (spec.layout == LayeredSpec::SEQUENTIAL) return forward_sequential(r, p);
     if (spec.layout == LayeredSpec::SCALED) return forward_scaled(r, p);
+    if (spec.layout == LayeredSpec::JOINT) return forward_joint(r, p);
     const kl::Batch &b = p.b;
     const int32_t *d_want = p.d_want;
     const int64_t T = p.T, R = p.R, max_ctx = p.max_ctx;

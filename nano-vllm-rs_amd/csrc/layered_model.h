@@ -12,7 +12,14 @@
 //                          positions added to the embedding; the mixer is an exponentially gated matrix memory (mLSTM), or a windowed attention (normed queries, keys
 //                          and values, query temperature, linear distance penalty, sink, output gate) side by side with an elementwise gated recurrence (minGRU),
 //                          each branch normed, half their sum; the feed-forward is dense with a squared ReLU; a layer may use an earlier layer's weights with a
-//                          cache / state of its own (layered_scaled.cpp).
+//                          cache / state of its own.
+//   joint (Sokalorn)     — x <- x + mixer(shift(n(x))) + ff(n(x)): ONE RMS norm per layer, read as it is by the feed-forward and through a token shift (a learned blend
+//                          with the previous token's norm output) by the mixer; the mixer is a state-space layer (causal convolution, step sizes, a decay per head,
+//                          input and output maps shared by groups of heads, gated group norm) or an attention without softmax (rotated queries and keys, capped scores,
+//                          chunks of positions, sigmoid weights with a bias per head, output gate) side by side with a time-mixing recurrence (five shifted inputs, a
+//                          decay per token and key channel, a bonus for the current token), each branch normed, half their sum; the feed-forward is a mixture of
+//                          clamped gated experts (softmax router, renormalised top-k, a gated shared expert); a range of layers runs several times with the same
+//                          weights, every pass starting with a product over [x ; embedding output] (layered_joint.cpp).
 //
 // The family shares the runner's step interface (sequences with a chunk [start, start + len) each: whole prompts, portions of prompts and
 // single decoded tokens in one batch), the block manager's tables (K/V pages) and state slots (recurrent state, convolution history), the
@@ -22,6 +29,7 @@
 #include <map>
 #include <string>
 #include <vector>
+#include "common.h"
 #include "json.h"
 #include "sequence.h"
 #include "kernels/layered.h"
@@ -31,9 +39,9 @@ struct nvr_model_runner;
 namespace nvr {
 
 struct LayeredSpec {
-    enum Mixer { ATTENTION = 0, RETENTION = 1, LATENT = 2, GLA = 3, MLSTM = 4, ATTN_GRU = 5 };
-    enum Ff { FF_NONE = 0, FF_CLAMPED_GLU = 1, FF_POLY = 2, FF_MOE = 3, FF_RELU2 = 4 };
-    enum Layout { PARALLEL = 0, SEQUENTIAL = 1, SCALED = 2 };
+    enum Mixer { ATTENTION = 0, RETENTION = 1, LATENT = 2, GLA = 3, MLSTM = 4, ATTN_GRU = 5, SSM = 6, ATTN_TMIX = 7 };
+    enum Ff { FF_NONE = 0, FF_CLAMPED_GLU = 1, FF_POLY = 2, FF_MOE = 3, FF_RELU2 = 4, FF_MOE_GLU = 5 };
+    enum Layout { PARALLEL = 0, SEQUENTIAL = 1, SCALED = 2, JOINT = 3 };
     struct Layer {
         int mixer = ATTENTION;
         int64_t heads = 0, kv_heads = 0, dim = 0, vdim = 0;
@@ -52,6 +60,14 @@ struct LayeredSpec {
         int64_t weights_of = -1;                            // the layer whose tensors this layer uses (-1: its own)
         int ff_kind = FF_NONE;
         int64_t experts = 0, top = 0, expert_ff = 0, shared_ff = 0;   // mixture of experts (shared_ff 0: no shared expert)
+        double shared_limit = 0.0;                          // clamped gated experts: the shared expert's limit (the routed experts' is `limit`)
+        // state-space mixer: heads x vdim channels, a state of dim x vdim per head, kv_heads groups of input / output maps; taps of its causal convolution and
+        // the parts of its gated norm
+        int64_t conv_taps = 1, mix_norm_groups = 1;
+        // attention over chunks without softmax: position i sees j <= i with floor(j / chunk) == floor(i / chunk); scores capped at softcap (0: not); the rotation's
+        // frequencies are divided by rot_factor
+        int64_t chunk = 0; double softcap = 0.0, rot_factor = 1.0;
+        int64_t t_heads = 0, t_dim = 0;                     // the time-mixing recurrence beside the attention: heads of t_dim x t_dim states
     };
     int layout = PARALLEL;
     int64_t norm_groups = 1;                                // sequential layout: RMS norms over this many equal parts of a row
@@ -63,10 +79,12 @@ struct LayeredSpec {
     int64_t taps = 1;                                       // causal convolution in front of every sublayer (1: a pointwise gain)
     std::vector<Layer> layers;
     std::vector<int> runs;                                  // layer index of every layer run, in order (loops unrolled)
+    std::vector<char> pass_start;                           // joint layout: this run starts a pass over the looped range (x <- W_loop [x ; embedding output] in front of it)
     bool stateful() const { return true; }                  // convolution history, and recurrent state where there is retention
     static int parse_rugudra(const Json &cfg, LayeredSpec *out);   // (model_registry.cpp)
     static int parse_pusunex(const Json &cfg, LayeredSpec *out);
     static int parse_sosutar(const Json &cfg, LayeredSpec *out);
+    static int parse_sokalorn(const Json &cfg, LayeredSpec *out);
 };
 
 class LayeredModel {
@@ -100,8 +118,17 @@ public:
         float *qn = nullptr, *kn = nullptr, *slope = nullptr;                        // attention: norm weights over the whole q / k projection; distance slopes [H]
         int64_t zcol = 0, ucol = 0, rgcol = 0;                                       // gated recurrence: columns of z, x and its gate in the mix projection
         void *wo2 = nullptr; float *bz = nullptr, *bu = nullptr, *outl = nullptr, *outr = nullptr;   // [W][gru_width]; biases [gru_width]; the branches' norms [W]
+        // joint layout
+        float *shift = nullptr;                                                      // [W] token shift in front of the mixer
+        float *convw = nullptr, *convb = nullptr, *dtb = nullptr, *alog = nullptr, *skip = nullptr;   // state-space mixer: [C][taps], [C], [H], [H], [H]
+        int64_t ccol = 0, dtcol = 0, conv_c = 0;                                     // columns of the convolved channels and of the step sizes in the mix projection
+        float *pb = nullptr; float *mu = nullptr;                                    // attention's bias per head; the five mixes' blends [5][W]
+        void *w4 = nullptr, *w1 = nullptr, *w2 = nullptr; int64_t t_rank = 0;         // time mixing: r / k / v / g stacked [4][Ht Dt][W]; decay projections [rank][W], [Ht Dt][rank]
+        float *w0 = nullptr, *bonus = nullptr, *tnorm = nullptr;                      // [Ht Dt] each
+        float *router2 = nullptr;                                                    // [E + 1][W] f32: the router's rows, then the shared expert's gate
     };
-    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; void *rows = nullptr; float *mstate = nullptr; };   // mstate: a matrix memory's running maxima [slots][H]   // borrowed: another run's pages (a shared latent)
+    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; void *rows = nullptr; float *mstate = nullptr;
+                      float *shist = nullptr, *chist = nullptr; };   // joint layout: hist the norm output before the step [2][slots][W], shist the mixer input's (time mixing), chist the convolution's inputs   // mstate: a matrix memory's running maxima [slots][H]   // borrowed: another run's pages (a shared latent)
     std::vector<LayerW> lw;
     std::vector<RunState> rs;
     void *embed = nullptr, *head = nullptr; float gfinal = 1.f;
@@ -115,6 +142,10 @@ public:
     void *pos = nullptr; void *tmp2 = nullptr, *gy = nullptr; float *gpre = nullptr, *tokg = nullptr, *gfloor = nullptr;   // [positions][W]; second branch's output, the recurrence's output; gates
     void *e_x = nullptr;                                                    // experts' inputs gathered in the order of the grouped rows
     void *e_gu = nullptr, *e_act = nullptr, *e_y = nullptr; int32_t *moe_i = nullptr; float *moe_score = nullptr;
+    // joint layout
+    void *loop_in = nullptr, *pair = nullptr; float *x0 = nullptr;          // [W][2 W]; [max tokens][2 W] operand rows; the embedding output
+    void *conv_o = nullptr, *mixes = nullptr, *tproj = nullptr, *tlow = nullptr, *tz = nullptr, *tcat = nullptr; float *shared_g = nullptr;
+    int64_t tlow_cap = 0;
     std::vector<void *> owned;                                              // device allocations of the sequential layout (freed with the model)
     // activations
     float *x = nullptr, *ret_o = nullptr;                                  // residual stream, retention outputs: f32
@@ -147,10 +178,20 @@ private:
     int init_scaled(nvr_model_runner &r);
     int load_scaled(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data);
     int forward_scaled(nvr_model_runner &r, const StepPlan &p);
+    int init_joint(nvr_model_runner &r);
+    int load_joint(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data);
+    int forward_joint(nvr_model_runner &r, const StepPlan &p);
     template <class T> int own(T **p, size_t bytes);
     int gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32 = false);
     int put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t rows, int64_t cols, int dtype, const void *src, bool as_operand);
 };
+
+template <class T> int LayeredModel::own(T **p, size_t bytes) {            // zeroed device memory that lives as long as the model
+    NVR_HIP_CHECK(hipMalloc((void **)p, bytes ? bytes : 16));
+    owned.push_back((void *)*p);
+    NVR_HIP_CHECK(hipMemset(*p, 0, bytes ? bytes : 16));
+    return NVR_OK;
+}
 
 }  // namespace nvr
 

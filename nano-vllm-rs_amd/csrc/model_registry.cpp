@@ -65,12 +65,18 @@ int parse_sosutar_spec(const Json &c, nvr_model_spec *out) {
     return LayeredSpec::parse_sosutar(c, &out->layered);
 }
 
+int parse_sokalorn_spec(const Json &c, nvr_model_spec *out) {
+    out->family = 1;
+    return LayeredSpec::parse_sokalorn(c, &out->layered);
+}
+
 struct Entry { const char *name; int (*parse)(const Json &, nvr_model_spec *); };
 const Entry kRegistry[] = {
     {"Qwen3ForCausalLM", parse_qwen3},
     {"Rugudra", parse_rugudra_spec},
     {"Pusunex", parse_pusunex_spec},
     {"Sosutar", parse_sosutar_spec},
+    {"Sokalorn", parse_sokalorn_spec},
 };
 
 }  // namespace
@@ -289,6 +295,85 @@ int LayeredSpec::parse_sosutar(const Json &c, LayeredSpec *s) {
         if (src[(size_t)i] != i) s->layers[(size_t)i].weights_of = src[(size_t)i];
         s->runs.push_back((int)src[(size_t)i]);
     }
+    return NVR_OK;
+}
+
+// Sokalorn: x <- x + mixer(shift(n(x))) + ff(n(x)) with one RMS norm per layer; mixers 'mamba2' (mixer.{heads, vdim, state, groups, conv, norm_groups}) and 'parallel'
+// (mixer.left: attention with rot.{dims, base, scaling.factor}, scale, softcap, mask.size — a chunk —, sigmoid weights; mixer.right: time mixing with heads x dim);
+// feed-forward 'moe' (expert.{ff, limit}, router.{experts, top}, optional shared.{ff, limit}) or none; 'loop': layers start .. stop-1 run `times` times, every pass
+// behind a product over [x ; embedding output].
+int LayeredSpec::parse_sokalorn(const Json &c, LayeredSpec *s) {
+    Reader rd;
+    s->layout = JOINT; s->taps = 1; s->residual_mult = 1.0; s->norm_groups = 1; s->embedding_scale = 1.0;
+    s->vocab = rd.integer(c, "vocab", ""); s->width = rd.integer(c, "width", "");
+    if (const Json *n = rd.need(c, "norm", "")) s->eps = rd.num(*n, "eps", "norm.");
+    const Json *layers = rd.need(c, "layers", "");
+    if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+    if (layers->kind != Json::Arr || layers->arr.empty()) return fail(NVR_ERR_INVALID_ARG, "config: 'layers' is not a list of layers");
+    if (s->vocab < 1 || s->width < 1) return fail(NVR_ERR_INVALID_ARG, "config: vocab and width must be positive");
+    s->layers.clear(); s->runs.clear(); s->pass_start.clear();
+    for (size_t i = 0; i < layers->arr.size(); ++i) {
+        const Json &lj = layers->arr[i];
+        const std::string w = "layers[" + std::to_string(i) + "].", wm = w + "mixer.";
+        Layer L;
+        const Json *type = rd.need(lj, "type", w), *mx = rd.need(lj, "mixer", w);
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (type->kind != Json::Str) return fail(NVR_ERR_INVALID_ARG, "config: '%stype' is not a string", w.c_str());
+        if (type->str == "mamba2") {
+            L.mixer = SSM;
+            L.heads = rd.integer(*mx, "heads", wm); L.vdim = rd.integer(*mx, "vdim", wm); L.dim = rd.integer(*mx, "state", wm); L.kv_heads = rd.integer(*mx, "groups", wm);
+            L.conv_taps = rd.integer(*mx, "conv", wm); L.mix_norm_groups = rd.integer(*mx, "norm_groups", wm);
+            if (rd.err.empty() && (L.conv_taps < 1 || L.mix_norm_groups < 1 || L.heads < 1 || L.vdim < 1 || (L.heads * L.vdim) % L.mix_norm_groups))
+                return fail(NVR_ERR_INVALID_ARG, "config: %s conv must be positive and norm_groups must divide heads * vdim", wm.c_str());
+        } else if (type->str == "parallel") {
+            L.mixer = ATTN_TMIX;
+            const Json *lf = rd.need(*mx, "left", wm), *rt = rd.need(*mx, "right", wm);
+            if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+            const std::string wl = wm + "left.";
+            L.heads = rd.integer(*lf, "heads", wl); L.kv_heads = rd.integer(*lf, "kv_heads", wl); L.dim = rd.integer(*lf, "dim", wl); L.vdim = rd.integer(*lf, "vdim", wl);
+            L.scale = rd.num(*lf, "scale", wl);
+            const Json *cap = lf->get("softcap");
+            if (cap && !cap->is_null()) L.softcap = rd.num(*lf, "softcap", wl);
+            const Json *mask = lf->get("mask");
+            if (mask && !mask->is_null()) L.chunk = rd.integer(*mask, "size", wl + "mask.");
+            const Json *rot = lf->get("rot");
+            if (rot && !rot->is_null()) {
+                L.rot_dims = rd.integer(*rot, "dims", wl + "rot."); L.rot_base = rd.num(*rot, "base", wl + "rot.");
+                const Json *sc = rot->get("scaling");
+                if (sc && !sc->is_null()) L.rot_factor = rd.num(*sc, "factor", wl + "rot.scaling.");
+            }
+            L.t_heads = rd.integer(*rt, "heads", wm + "right."); L.t_dim = rd.integer(*rt, "dim", wm + "right.");
+            if (rd.err.empty() && (L.chunk < 0 || L.softcap < 0 || L.rot_dims < 0 || L.rot_dims % 2 || L.rot_dims > L.dim || !(L.rot_factor > 0) || L.t_heads < 1 || L.t_dim < 1))
+                return fail(NVR_ERR_INVALID_ARG, "config: %s needs an even rot.dims <= dim, a positive scaling factor and positive right.heads / right.dim", wm.c_str());
+        } else return fail(NVR_ERR_UNSUPPORTED, "config: layer type '%s' (mamba2 or parallel)", type->str.c_str());
+        const Json *mlp = lj.get("mlp");
+        if (mlp && !mlp->is_null()) {
+            const Json *kind = rd.need(*mlp, "kind", w + "mlp.");
+            if (kind && !(kind->kind == Json::Str && kind->str == "moe")) return fail(NVR_ERR_UNSUPPORTED, "config: '%smlp.kind' (moe)", w.c_str());
+            L.has_mlp = true; L.ff_kind = FF_MOE_GLU;
+            const Json *ex = rd.need(*mlp, "expert", w + "mlp."), *ro = rd.need(*mlp, "router", w + "mlp."), *sh = mlp->get("shared");
+            if (ex) { L.expert_ff = rd.integer(*ex, "ff", w + "mlp.expert."); L.limit = rd.num(*ex, "limit", w + "mlp.expert."); }
+            if (ro) { L.experts = rd.integer(*ro, "experts", w + "mlp.router."); L.top = rd.integer(*ro, "top", w + "mlp.router."); }
+            if (sh && !sh->is_null()) { L.shared_ff = rd.integer(*sh, "ff", w + "mlp.shared."); L.shared_limit = rd.num(*sh, "limit", w + "mlp.shared."); }
+            if (rd.err.empty() && (L.expert_ff < 1 || L.experts < 1 || L.top < 1 || L.top > L.experts || L.shared_ff < 0))
+                return fail(NVR_ERR_INVALID_ARG, "config: %smlp needs positive expert sizes and 1 <= top <= experts", w.c_str());
+        }
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (L.heads < 1 || L.dim < 1 || L.vdim < 1 || L.kv_heads < 1 || L.heads % L.kv_heads)
+            return fail(NVR_ERR_INVALID_ARG, "config: %s %ld heads over %ld groups of %ld / %ld", w.c_str(), (long)L.heads, (long)L.kv_heads, (long)L.dim, (long)L.vdim);
+        s->layers.push_back(L);
+    }
+    const int64_t n = (int64_t)s->layers.size();
+    const Json *loop = c.get("loop");
+    if (loop && !loop->is_null()) {
+        const int64_t a = rd.integer(*loop, "start", "loop."), b = rd.integer(*loop, "stop", "loop."), t = rd.integer(*loop, "times", "loop.");
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (a < 0 || b < a || b > n || t < 1) return fail(NVR_ERR_INVALID_ARG, "config: loop [%ld, %ld) x %ld over %ld layers", (long)a, (long)b, (long)t, (long)n);
+        for (int64_t i = 0; i < a; ++i) { s->runs.push_back((int)i); s->pass_start.push_back(0); }
+        for (int64_t k = 0; k < t; ++k) for (int64_t i = a; i < b; ++i) { s->runs.push_back((int)i); s->pass_start.push_back(i == a ? 1 : 0); }
+        for (int64_t i = b; i < n; ++i) { s->runs.push_back((int)i); s->pass_start.push_back(0); }
+    } else
+        for (int64_t i = 0; i < n; ++i) { s->runs.push_back((int)i); s->pass_start.push_back(0); }
     return NVR_OK;
 }
 
