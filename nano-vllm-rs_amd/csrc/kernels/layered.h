@@ -56,7 +56,7 @@ struct SinkAttnArgs {
     int32_t chunk;                           // > 0: position i sees only the keys j <= i of its own chunk, floor(j / chunk) == floor(i / chunk), chunks counted from position 0
     float softcap;                           // > 0: score <- softcap * tanh(score / softcap) (after the scale, before any bias)
     const float *gate_bias;                  // not null: no softmax — the weight of a visible key is sigmoid(score + gate_bias[h]), not normalised over the keys
-                                             // (general form and gate_attention_tiled; not together with a penalty or a sink)
+                                             // (both forms; not together with a penalty or a sink)
 };
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);     // any shape; a context that fits the LDS score buffer
 // The same on the matrix cores (bf16 operands, D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16).  tiles (device, built by the host): tile i covers the
@@ -231,7 +231,7 @@ int scale_f32(float *y, int64_t n, float c, hipStream_t s);
 // ---------------------------------------------------------------------------------------------------------------------------------------------------
 // Blocks of layers whose two sublayers read ONE norm, with a token shift in front of the mixer (layered_ssm.hip): a state-space mixer (causal convolution, step
 // sizes, gated group norm; its recurrence is retention's token-gated form with shared input / output maps), rotated keys on their way into the pages, an
-// attention without softmax over chunks of positions, the mixes of a time-mixing recurrence (retention's gated form with a bonus), the input of a pass over a
+// attention without softmax over chunks of positions (SinkAttnArgs::gate_bias, chunk, softcap in both attention forms), the mixes of a time-mixing recurrence (retention's gated form with a bonus), the input of a pass over a
 // looped range of layers.
 
 // h = x / sqrt(mean(x^2) + eps) * w -> out_h (may be null); m_t = h_t + (h_(t-1) - h_t) * shift -> out_m (operand type; h_(-1) = 0; the row before a chunk comes from
@@ -264,10 +264,5 @@ int shift_mixes(const void *m, int64_t ldm, const Batch &b, int64_t W, int32_t n
 
 // y = tanh(y) in place (rows of N numbers, stride ld)
 int tanh_rows(void *y, int64_t ld, int64_t T, int64_t N, bool bf16, hipStream_t s);
-
-// Attention without softmax on the matrix cores (bf16 operands; gate_bias set; D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16): the tiles of sink_attention_tiled,
-// P = sigmoid(capped score + bias) on the visible keys of the row's chunk, O = P V summed over the key tiles.
-bool gate_attention_tiled_ok(const SinkAttnArgs &a, bool bf16, int block_size);
-int gate_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, hipStream_t s);
 
 }}  // namespace nvr::kl

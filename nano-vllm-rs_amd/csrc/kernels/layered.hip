@@ -291,7 +291,9 @@ __global__ __launch_bounds__(256) void penalty_table_kernel(const float *__restr
     if (d < n) tab[(int64_t)h * n + d] = (r2 ? r1[h] * log1pf(r2[h] * (float)d) : r1[h] * (float)d) * kLog2e;      // (r2 null: linear in the distance)
 }
 
-template <int C>
+// GATE: no softmax — the weight of a visible key is sigmoid(capped score + bias of the head), the tiles' products are summed as they are (a split's partial carries
+// m = 0 and the first split l = 1, so that the merge adds the partials up).  chunk > 0 (both forms): a row sees the keys from its chunk's first position on.
+template <int C, bool GATE = false>
 __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, Batch b, const AttnTile *__restrict__ tiles, int nsplit, float *__restrict__ part_o,
                                                              float *__restrict__ part_ml) {
     constexpr int KT = 64, KS = C + 8, VS = KT + 8, VG = C + 1, NCH = C / 32;   // NCH: 16-byte pieces of a K (or V) tile per thread
@@ -320,14 +322,16 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
 #pragma unroll
         for (int ks = 0; ks < C / 32; ++ks) if (ks < d32) qf[ks] = *reinterpret_cast<const bf16x8 *>(q + ks * 32);
     }
-    int pos[4], hgi[4]; float m[4], l[4];
+    int pos[4], hgi[4], cs[4]; float m[4], l[4], gb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int r = wave * 16 + lq * 4 + i, h = kvh * g + r % g;
         pos[i] = st + lr0 + r / g; hgi[i] = r % g;
+        cs[i] = a.chunk > 0 ? pos[i] / a.chunk * a.chunk : 0;      // first key of the row's chunk
         const bool sink_here = a.sink && z == 0;
-        m[i] = sink_here ? a.sink[h] * kLog2e : -INFINITY;
-        l[i] = (sink_here && lm == 0) ? 1.f : 0.f;
+        m[i] = GATE ? 0.f : sink_here ? a.sink[h] * kLog2e : -INFINITY;
+        l[i] = ((GATE || sink_here) && z == 0 && lm == 0) ? 1.f : 0.f;
+        gb[i] = GATE ? a.gate_bias[h] : 0.f;
     }
     f32x4 acc[C / 16];
 #pragma unroll
@@ -336,7 +340,8 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
     const int p0 = st + lr0;                            // first position of the tile
     const int nkeys = p0 + npos;                        // keys the tile's last position sees
     const int ntl = (nkeys + KT - 1) / KT;
-    const int kt0 = a.window > 0 ? max(p0 - a.window + 1, 0) / KT : 0;      // first key tile the tile's first position can see
+    int kt0 = a.window > 0 ? max(p0 - a.window + 1, 0) / KT : 0;            // first key tile the tile's first position can see
+    if (a.chunk > 0) kt0 = max(kt0, p0 / a.chunk * a.chunk / KT);
     const int kch = D >> 3;
     uint4 kreg[NCH], vreg[NCH];
     // a thread's pieces: key skey, 16-byte pieces sch, sch + 4, ... of its row; key group vkg, columns vcl, vcl + 32, ... (one block-table lookup each per tile)
@@ -389,6 +394,21 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
                         s[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, s[nt], 0, 0, 0);
                     }
             }
+            if (GATE) {
+                const float c2 = a.softcap > 0.f ? 2.0f * kLog2e / a.softcap : 0.f;
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const int j = k0 + nt * 16 + lm;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float v = s[nt][i] * a.scale;
+                        if (a.softcap > 0.f) v = a.softcap * (1.0f - 2.0f / (exp2f(v * c2) + 1.0f));      // cap * tanh(v / cap)
+                        const float p = (j > pos[i] || j < cs[i]) ? 0.f : 1.0f / (1.0f + exp2f(-kLog2e * (v + gb[i])));
+                        const __bf16 pb = (__bf16)p;
+                        Ps[(wave * 16 + lq * 4 + i) * VS + nt * 16 + lm] = __builtin_bit_cast(bf16_t, pb);
+                    }
+                }
+            } else {
             float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
@@ -398,7 +418,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
                     const int dist = pos[i] - j;
                     float v = s[nt][i] * scale2;
                     if (a.pen) v -= pen[(hgi[i] << 7) + min(max(dist - dmin, 0), 127)];
-                    v = (dist < 0 || (a.window > 0 && dist >= a.window)) ? -INFINITY : v;
+                    v = (dist < 0 || (a.window > 0 && dist >= a.window) || j < cs[i]) ? -INFINITY : v;
                     s[nt][i] = v;
                     mx[i] = fmaxf(mx[i], v);
                 }
@@ -422,6 +442,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
                 l[i] = l[i] * alpha + rs;
 #pragma unroll
                 for (int t = 0; t < C / 16; ++t) acc[t][i] *= alpha;
+            }
             }
             __builtin_amdgcn_wave_barrier();                // (the weights are read back by this wave only: LDS serves a wave's requests in order)
 #pragma unroll
@@ -831,6 +852,9 @@ int prepare() {
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<256>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<64, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<128, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<256, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)norm_canon_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)norm_canon_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     return 0;
@@ -894,7 +918,12 @@ int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *
     const int C = std::max(a.D, a.Dv) <= 64 ? 64 : std::max(a.D, a.Dv) <= 128 ? 128 : 256;
     const size_t lds = ((size_t)64 * (C + 8) + (size_t)8 * (C + 1) * 8 + (size_t)64 * 72) * 2 + (size_t)(a.H / a.G) * 128 * 4;
     const dim3 grid((unsigned)ntiles, (unsigned)a.G, (unsigned)nsplit);
-    if (C == 64) sink_attn_mfma_kernel<64><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
+    if (a.gate_bias) {
+        if (a.r1 || a.r2 || a.slope || a.sink || a.pen) return nvr::fail(NVR_ERR_INVALID_ARG, "sink_attention_tiled: gated weights take no penalty and no sink");
+        if (C == 64) sink_attn_mfma_kernel<64, true><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
+        else if (C == 128) sink_attn_mfma_kernel<128, true><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
+        else sink_attn_mfma_kernel<256, true><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
+    } else if (C == 64) sink_attn_mfma_kernel<64><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
     else if (C == 128) sink_attn_mfma_kernel<128><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
     else sink_attn_mfma_kernel<256><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
     if (int rc = launched("sink_attention_tiled")) return rc;

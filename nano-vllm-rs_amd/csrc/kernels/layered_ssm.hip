@@ -1,7 +1,6 @@
 // layered_ssm.hip — blocks of layers whose two sublayers read one norm, with a token shift in front of the mixer (kernels/layered.h): the norm with the shift, the
 // input of a pass over a looped range, the front (causal convolution, step sizes) and the end (skip, gate, group norm) of a state-space mixer whose recurrence is
-// retention's token-gated form, rotated queries and keys on their way into the pages, the mixes of a time-mixing recurrence, and an attention without softmax over
-// chunks of positions on the matrix cores.  Norms, angles, step sizes, decays and scores are f32 in both operand types.  wave64, gfx950.
+// retention's token-gated form, rotated queries and keys on their way into the pages, the mixes of a time-mixing recurrence.  Norms, angles, step sizes, decays and scores are f32 in both operand types.  wave64, gfx950.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <algorithm>
@@ -250,8 +249,5 @@ int tanh_rows(void *y, int64_t ld, int64_t T, int64_t N, bool bf16, hipStream_t 
     else tanh_rows_kernel<float><<<grid, dim3(256), 0, s>>>((float *)y, ld, T, N);
     return launched("tanh_rows");
 }
-
-bool gate_attention_tiled_ok(const SinkAttnArgs &, bool, int) { return false; }
-int gate_attention_tiled(const SinkAttnArgs &, const Batch &, const AttnTile *, int, hipStream_t) { return nvr::fail(NVR_ERR_UNSUPPORTED, "gate_attention_tiled: not built"); }
 
 }}  // namespace nvr::kl

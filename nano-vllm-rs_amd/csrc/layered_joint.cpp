@@ -25,8 +25,7 @@ int LayeredModel::init_joint(nvr_model_runner &r) {
     };
     lw.resize(spec.layers.size());
     int64_t max_nmix = 0, max_cat = 0, max_ro = 0, max_conv = 0, max_h = 1, max_t4 = 0, max_tn = 0, max_fs = 0, max_top = 0, max_e2f = 0, max_ef = 0, max_experts = 0, max_f = 0;
-    bool loops = false;
-    for (char c : spec.pass_start) loops = loops || c;
+    const bool loops = spec.has_loop;
     for (size_t i = 0; i < spec.layers.size(); ++i) {
         const LayeredSpec::Layer &L = spec.layers[i]; LayerW &w = lw[i];
         RC(own(&w.n1, (size_t)W * 4)); RC(own(&w.shift, (size_t)W * 4));
@@ -50,7 +49,7 @@ int LayeredModel::init_joint(nvr_model_runner &r) {
             if (std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) == attn_groups.end()) attn_groups.push_back(L.heads / L.kv_heads);
             max_cat = std::max(max_cat, hv); max_ro = std::max(max_ro, tn); max_t4 = std::max(max_t4, 4 * tn); max_tn = std::max(max_tn, tn);
         } else return fail(NVR_ERR_UNSUPPORTED, "layer %zu: this mixer does not belong to the joint layout", i);
-        RC(own(&w.mix, (size_t)(w.nmix * W * esz)));
+        RC(named(&w.mix, (size_t)(w.nmix * W * esz)));         // (freed by name with the model)
         if (L.ff_kind == LayeredSpec::FF_MOE_GLU) {
             const int64_t f = L.expert_ff, fs = L.shared_ff;
             RC(own(&w.router2, (size_t)((L.experts + 1) * W) * 4));
@@ -242,13 +241,17 @@ int LayeredModel::forward_joint(nvr_model_runner &r, const StepPlan &p) {
             a.q = at(proj, w.qcol); a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.chunk = (int32_t)L.chunk; a.softcap = (float)L.softcap; a.gate_bias = w.pb;
             a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale; a.out = cat; a.ldo = hv;
             a.v_grouped = 1;
-            const bool tiled = kl::gate_attention_tiled_ok(a, bf16, (int)r.block_size);       // (a property of the layer's shape: the pages keep one layout)
+            const bool tiled = kl::sink_attention_tiled_ok(a, bf16, (int)r.block_size);       // (a property of the layer's shape: the pages keep one layout)
             kl::RopeStoreArgs ra{}; ra.proj = proj; ra.ld = w.nmix; ra.qcol = w.qcol; ra.kcol = w.kcol; ra.vcol = w.vcol; ra.H = a.H; ra.G = a.G; ra.D = a.D; ra.Dv = a.Dv;
             ra.rot = (int32_t)L.rot_dims; ra.freq = w.rfreq; ra.kc = st.kc; ra.vc = st.vc; ra.v_grouped = tiled;
             RC(kl::rope_store(ra, b, bf16, s));
             if (tiled) {
                 const size_t gi = (size_t)(std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) - attn_groups.begin());
-                RC(kl::gate_attention_tiled(a, b, (const kl::AttnTile *)(in_dev + p.o_tiles[gi]), p.n_tiles[gi], s));
+                // decode-sized steps over long chunks: few tiles, many keys each — a tile's keys go to several workgroups whose partial sums are added up
+                const int64_t wgs = (int64_t)p.n_tiles[gi] * L.kv_heads, keys = L.chunk > 0 ? std::min<int64_t>(p.max_ctx, L.chunk + 64) : p.max_ctx;
+                int64_t nsplit = 1;
+                if (wgs < r.num_cus && keys >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / wgs, (keys + 255) / 256, 16}));
+                RC(kl::sink_attention_tiled(a, b, (const kl::AttnTile *)(in_dev + p.o_tiles[gi]), p.n_tiles[gi], (int)nsplit, attn_ws, attn_ws_bytes, s));
             } else
                 RC(kl::sink_attention(a, b, bf16, s));
             RC(kl::sigmoid_gate(cat, hv, at(proj, w.gcol), w.nmix, T, hv, bf16, s));

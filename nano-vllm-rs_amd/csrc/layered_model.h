@@ -79,6 +79,7 @@ struct LayeredSpec {
     int64_t taps = 1;                                       // causal convolution in front of every sublayer (1: a pointwise gain)
     std::vector<Layer> layers;
     std::vector<int> runs;                                  // layer index of every layer run, in order (loops unrolled)
+    bool has_loop = false;                                  // joint layout: the configuration names a looped range (the checkpoint then holds its input product, used or not)
     std::vector<char> pass_start;                           // joint layout: this run starts a pass over the looped range (x <- W_loop [x ; embedding output] in front of it)
     bool stateful() const { return true; }                  // convolution history, and recurrent state where there is retention
     static int parse_rugudra(const Json &cfg, LayeredSpec *out);   // (model_registry.cpp)

@@ -311,7 +311,7 @@ int LayeredSpec::parse_sokalorn(const Json &c, LayeredSpec *s) {
     if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
     if (layers->kind != Json::Arr || layers->arr.empty()) return fail(NVR_ERR_INVALID_ARG, "config: 'layers' is not a list of layers");
     if (s->vocab < 1 || s->width < 1) return fail(NVR_ERR_INVALID_ARG, "config: vocab and width must be positive");
-    s->layers.clear(); s->runs.clear(); s->pass_start.clear();
+    s->layers.clear(); s->runs.clear(); s->pass_start.clear(); s->has_loop = false;
     for (size_t i = 0; i < layers->arr.size(); ++i) {
         const Json &lj = layers->arr[i];
         const std::string w = "layers[" + std::to_string(i) + "].", wm = w + "mixer.";
@@ -369,6 +369,7 @@ int LayeredSpec::parse_sokalorn(const Json &c, LayeredSpec *s) {
         const int64_t a = rd.integer(*loop, "start", "loop."), b = rd.integer(*loop, "stop", "loop."), t = rd.integer(*loop, "times", "loop.");
         if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
         if (a < 0 || b < a || b > n || t < 1) return fail(NVR_ERR_INVALID_ARG, "config: loop [%ld, %ld) x %ld over %ld layers", (long)a, (long)b, (long)t, (long)n);
+        s->has_loop = true;
         for (int64_t i = 0; i < a; ++i) { s->runs.push_back((int)i); s->pass_start.push_back(0); }
         for (int64_t k = 0; k < t; ++k) for (int64_t i = a; i < b; ++i) { s->runs.push_back((int)i); s->pass_start.push_back(i == a ? 1 : 0); }
         for (int64_t i = b; i < n; ++i) { s->runs.push_back((int)i); s->pass_start.push_back(0); }

@@ -155,9 +155,13 @@ def clamped_expert(h, wt, p, limit):
     return (g * sigmoid(1.702 * g) * (u + 1.0)) @ wt[p + "down"].T
 
 
-def route(h, wt, p, top):
-    """Softmax over all experts; the `top` largest; their scores divided by their sum.  Returns (chosen [T, top], weights [T, top])."""
+def route(h, wt, p, top, margins=None):
+    """Softmax over all experts; the `top` largest; their scores divided by their sum.  Returns (chosen [T, top], weights [T, top]).
+    margins (a list) collects, per token, the gap between the last chosen and the first rejected logit."""
     z = h @ wt[p + "router"].T
+    if margins is not None and top < z.shape[1]:
+        zs = np.sort(z, axis=-1)[:, ::-1]
+        margins.extend((zs[:, top - 1] - zs[:, top]).tolist())
     z = z - z.max(axis=-1, keepdims=True)
     s = np.exp(z)
     s /= s.sum(axis=-1, keepdims=True)
@@ -166,9 +170,9 @@ def route(h, wt, p, top):
     return chosen, w / (w.sum(axis=-1, keepdims=True) + 1e-20)
 
 
-def expert_ff(h, f, wt, p):
+def expert_ff(h, f, wt, p, margins=None):
     """Mixture of experts with an optional shared expert that every token uses, times sigmoid(W_sg h)."""
-    chosen, w = route(h, wt, p, f["router"]["top"])
+    chosen, w = route(h, wt, p, f["router"]["top"], margins)
     y = np.zeros((h.shape[0], wt[p + "e0.down"].shape[0]))
     for t in range(h.shape[0]):
         for c, wc in zip(chosen[t], w[t]):
@@ -189,7 +193,7 @@ def layer_runs(cfg):
     return runs + [(i, False) for i in range(loop["stop"], n)]
 
 
-def forward(cfg, wt, tokens, layer_outputs=None, pos0=0, states=None):
+def forward(cfg, wt, tokens, layer_outputs=None, pos0=0, states=None, margins=None):
     """Logits [T, vocab] of one sequence's tokens at positions pos0 ..; states: the list forward returned for the tokens before (None: a new
     sequence).  Returns (logits, states)."""
     eps = cfg["norm"]["eps"]
@@ -212,7 +216,7 @@ def forward(cfg, wt, tokens, layer_outputs=None, pos0=0, states=None):
             raise ValueError(L["type"])
         new_states.append((last, ms))
         if L.get("mlp") is not None:
-            y = y + expert_ff(h, L["mlp"], wt, p + "mlp.")
+            y = y + expert_ff(h, L["mlp"], wt, p + "mlp.", margins)
         x = x + y
         if layer_outputs is not None:
             layer_outputs.append(x.copy())
