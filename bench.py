@@ -700,10 +700,10 @@ def main() -> None:
                          "NVR_BENCH_LIVE_PMC=0 does the same): the committed pass under profiles/ is quoted instead")
     ap.add_argument("--layered-compare", action="store_true",
                     help="instead of the headline workload: prefill and decode throughput of the layer-list designs (Rugudra: attention with distance penalty and sink, "
-                         "retention, clamped gated feed-forward; Pusunex: latent attention, gated linear attention, experts; Sosutar: matrix memory, windowed attention beside a gated recurrence) beside the dense Qwen3 graph at equal "
+                         "retention, clamped gated feed-forward; Pusunex: latent attention, gated linear attention, experts; Sosutar: matrix memory, windowed attention beside a gated recurrence; Sokalorn: state-space mixer, chunked sigmoid attention beside time mixing, clamped experts) beside the dense Qwen3 graph at equal "
                          "layer sizes, random weights, one JSON line per size")
     ap.add_argument("--layered-sizes", default="w1024,w2048", help="sizes of --layered-compare (w1024, w2048, w4096)")
-    ap.add_argument("--layered-models", default="rugudra,qwen3", help="models of --layered-compare (rugudra, pusunex, sosutar, qwen3)")
+    ap.add_argument("--layered-models", default="rugudra,qwen3", help="models of --layered-compare (rugudra, pusunex, sosutar, sokalorn, qwen3)")
     args = ap.parse_args()
     if args.layered_compare:
         import importlib

@@ -44,6 +44,7 @@ struct FlashParams {
     const int32_t *srows, *scount;     // optional: only the rows srows[0 .. *scount) of the batch share the prefix (row srows[0] names its blocks)
     const float *r1, *r2, *sink; int64_t ldo;   // PEN instantiations: distance penalty and sink per head (FlashArgs); ldo: output row stride in elements
     int32_t window;                              // PEN instantiations: > 0, a query sees only the keys less than `window` positions back
+    const float *gate_bias; float softcap; int32_t chunk;   // GATE instantiations (FlashArgs): sigmoid weights with a bias per head, capped scores, chunks of positions
 };
 
 
@@ -123,7 +124,9 @@ constexpr int FLASH_WAVES = NVR_FLASH_WAVES;     // waves per workgroup: 32 quer
 // schedule — 128/G sequences per workgroup, no causal mask, every key of [0, shared_len) visible to every row — and the result
 // leaves as the split-KV partial of partition 0 (unnormalised f32 o, scaled max, sum), merged with the per-sequence remainder
 // by attn_merge_kernel.
-template <int D, int G, bool PAGED, bool UB = false, bool SHARED = false, bool PEN = false>
+// GATE: no softmax — a visible key's weight is sigmoid(cap tanh(score / cap) + bias of the head), not normalised; a query sees the keys of its own chunk of
+// p.chunk positions (chunks count from position 0) up to itself; the steps start at the chunk of the tile's first query.
+template <int D, int G, bool PAGED, bool UB = false, bool SHARED = false, bool PEN = false, bool GATE = false>
 __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefill_kernel(FlashParams p) {   // 2 waves per SIMD: <= 256 registers per lane
     constexpr int NT = 64 * FLASH_WAVES;         // threads
     constexpr int KT = NVR_FLASH_KT;             // keys per step
@@ -147,7 +150,8 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
     const int r = lane & 15, g4 = lane >> 4;
     // SHARED: blockIdx.y cuts the shared keys into partitions of shared_len tokens (more workgroups than 8 per kv head at 512 sequences)
     // (a window: the first step is the one that holds the first key the tile's first query sees)
-    const int kv_start = SHARED ? (int)blockIdx.y * p.shared_len : ((PEN && p.window > 0) ? max(tile.pos0 - p.window + 1, 0) / KT * KT : 0);
+    const int kv_start = SHARED ? (int)blockIdx.y * p.shared_len : ((PEN && p.window > 0) ? max(tile.pos0 - p.window + 1, 0) / KT * KT :
+                                                                    (GATE && p.chunk > 0) ? tile.pos0 / p.chunk * p.chunk / KT * KT : 0);
     const int kv_end = SHARED ? kv_start + p.shared_len : tile.pos0 + tile.nq;
 
     // the wave's two query tiles: head and position block
@@ -278,6 +282,10 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
     half8_t ones;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ones[e] = (half_t)1.0f;
+    float gbias[NQT], gcap2 = 0.f; int qcs[NQT];               // GATE: the head's bias, 2 log2(e) / cap, the first key of the query's chunk
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) { gbias[t] = GATE ? p.gate_bias[head[t]] : 0.f; qcs[t] = (GATE && p.chunk > 0) ? qpos[t] / p.chunk * p.chunk : 0; }
+    if (GATE && p.softcap > 0.f) gcap2 = 2.0f * 1.44269504088896340736f / p.softcap;
 
     const int nsteps = (kv_end - kv_start + KT - 1) / KT;
     // step `it` computes on ring slot it % NBUF while tile it+NBUF-1 is requested into the slot step it-1 just released;
@@ -315,6 +323,21 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
                 for (int t = 0; t < NQT; ++t) s[t][mt] = mfma16(kf[mt & 1][ks], qf[t][ks], s[t][mt]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        half8_t pf[NQT][NK2];
+        if (GATE) {
+#pragma unroll
+            for (int t = 0; t < NQT; ++t)
+#pragma unroll
+                for (int mt = 0; mt < NMT; ++mt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int j = kt + mt * 16 + g4 * 4 + e;
+                        float v = s[t][mt][e] * p.scale;
+                        if (p.softcap > 0.f) v = p.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(v * gcap2) + 1.0f));      // cap * tanh(v / cap)
+                        const float w = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * (v + gbias[t])));
+                        pf[t][mt >> 1][(mt & 1) * 4 + e] = (half_t)((j > qpos[t] || j < qcs[t]) ? 0.f : w);
+                    }
+        } else {
         if (PEN) {
 #pragma unroll
             for (int t = 0; t < NQT; ++t)
@@ -338,7 +361,6 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
                     for (int e = 0; e < 4; ++e)
                         if (kt + mt * 16 + g4 * 4 + e > qpos[t]) s[t][mt][e] = -INFINITY;
         }
-        half8_t pf[NQT][NK2];
         bool moved = false;
         float alpha[NQT];
 #pragma unroll
@@ -366,13 +388,16 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
                 for (int dt = 0; dt < NDT; ++dt) o[t][dt] *= alpha[t];
             }
         }
+        }   // !GATE
         // Oᵀ += Vᵀ·Pᵀ per 32-key half; one V fragment (two transposing reads) feeds both query tiles
 #pragma unroll
         for (int k2 = 0; k2 < NK2; ++k2) {
             const int row0 = (2 * k2) * 16 + g4 * 4 + (r >> 2), row1 = row0 + 16;
             const int sw = v_swz<D>(row0);                      // same for row1 (row1 = row0 + 16)
+            if (!GATE) {
 #pragma unroll
-            for (int t = 0; t < NQT; ++t) ol[t] = mfma16(ones, pf[t][k2], ol[t]);
+                for (int t = 0; t < NQT; ++t) ol[t] = mfma16(ones, pf[t][k2], ol[t]);
+            }
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) {
                 const int cb = ((((dt * 2 + ((r & 3) >> 1)) ^ sw) << 4) | ((r & 1) << 3));   // byte offset inside the row
@@ -429,7 +454,7 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
     for (int t = 0; t < NQT; ++t) {
         if (qvalid[t]) {
             const float ls = ol[t][0];                          // every row of the ones-product holds the query's sum
-            const float inv = ls > 0.f ? 1.0f / ls : 0.f;
+            const float inv = GATE ? 1.0f : ls > 0.f ? 1.0f / ls : 0.f;
             half_t *orow = p.out + (int64_t)qrow[t] * p.ldo + (int64_t)head[t] * D + g4 * 4;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) {
@@ -456,6 +481,9 @@ int flash_prefill(const FlashArgs &a, bool paged, hipStream_t s) {
     p.bs_shift = (a.block_size > 0 && (a.block_size & (a.block_size - 1)) == 0) ? __builtin_ctz(a.block_size) : -1;
     p.tiles = a.tiles; p.H = a.H; p.KVH = a.KVH; p.scale = a.scale; p.out = (half_t *)a.out;
     p.r1 = a.r1; p.r2 = a.r2; p.sink = a.sink; p.ldo = a.ldo ? a.ldo : (int64_t)a.H * a.D; p.window = a.window;
+    p.gate_bias = a.gate_bias; p.softcap = a.softcap; p.chunk = a.chunk;
+    const bool gate = a.gate_bias != nullptr;
+    if (gate && (a.r1 || a.sink || a.window > 0 || !paged)) return nvr::fail(NVR_ERR_UNSUPPORTED, "flash_prefill: gated weights take no penalty, sink or window and read K and V through block tables");
     const bool pen = a.r1 || a.sink;
     if (a.window > 0 && !a.sink) return nvr::fail(NVR_ERR_UNSUPPORTED, "flash_prefill: a window needs the sink form (a step may hold no visible key)");
     if (pen && !paged) return nvr::fail(NVR_ERR_UNSUPPORTED, "flash_prefill: the penalty / sink form reads K and V through block tables");
@@ -464,7 +492,9 @@ int flash_prefill(const FlashArgs &a, bool paged, hipStream_t s) {
     const bool ub = paged && p.bs_shift >= 0 && a.block_size % NVR_FLASH_KT == 0;
 #define NVR_FLASH(DD, GG)                                                                             \
     if (a.D == DD && G == GG) {                                                                       \
-        if (pen && ub) flash_prefill_kernel<DD, GG, true, true, false, true><<<grid, block, 0, s>>>(p);   \
+        if (gate && ub) flash_prefill_kernel<DD, GG, true, true, false, false, true><<<grid, block, 0, s>>>(p);   \
+        else if (gate) flash_prefill_kernel<DD, GG, true, false, false, false, true><<<grid, block, 0, s>>>(p);   \
+        else if (pen && ub) flash_prefill_kernel<DD, GG, true, true, false, true><<<grid, block, 0, s>>>(p);   \
         else if (pen) flash_prefill_kernel<DD, GG, true, false, false, true><<<grid, block, 0, s>>>(p);   \
         else if (ub) flash_prefill_kernel<DD, GG, true, true><<<grid, block, 0, s>>>(p);              \
         else if (paged) flash_prefill_kernel<DD, GG, true><<<grid, block, 0, s>>>(p);                 \

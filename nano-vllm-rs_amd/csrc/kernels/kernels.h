@@ -64,6 +64,9 @@ struct FlashArgs {
     // r1 without r2: a penalty linear in the distance, r1[h] * (i - j).  window > 0 (with a sink): a query sees only the keys less than `window` positions back.
     const float *r1, *r2, *sink; int64_t ldo;
     int32_t window;
+    // gate_bias ([H] f32 on the device; paged K / V; no penalty, sink or window): no softmax — a visible key's weight is sigmoid(score + gate_bias[h]) with the scaled
+    // score first capped, softcap * tanh(score / softcap) (softcap 0: not); chunk > 0: a query sees the keys j <= i with floor(j / chunk) == floor(i / chunk)
+    const float *gate_bias; float softcap; int32_t chunk;
 };
 
 // Config.dtype = "float32": attention arguments of the f32 path (kernels/f32_path.hip)

@@ -161,7 +161,8 @@ int silu_mul(const void *gu, int64_t T, int64_t F, void *out, int64_t ldo, bool 
 // softmax: score is the chosen experts' share of the softmax over ALL experts, divided by the sum of the chosen shares (+ 1e-20), instead of the sigmoid.
 // extra > 0: rows E .. E + extra - 1 of wr are further f32 projections of h that leave as they are in extra_out[t * extra + i] (a shared expert's gate).
 int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr, int64_t E, int64_t top, int32_t *sel, float *score, int32_t *off, int32_t *order,
-              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s, bool softmax = false, int64_t extra = 0, float *extra_out = nullptr);
+              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s, bool softmax = false, int64_t extra = 0, float *extra_out = nullptr,
+              const float *logits = nullptr, int64_t ldl = 0);   // logits (f32 rows of E + extra numbers, stride ldl): the products wr h formed beforehand (wr is then not read)
 int moe_gather(const void *h, int64_t ldh, int64_t T, int64_t W, int64_t top, const int32_t *place_of, const float *score, void *xs, bool bf16, hipStream_t s);
 // out[t] = sum_k y[place_of[t * top + k]] + shared[t] (shared may be null).  With score ([T][top] f32) choice k is weighted by score[t * top + k]; with shared_gate
 // ([T] f32, stride gate_ld) the shared row is multiplied by sigmoid(shared_gate[t * gate_ld]).

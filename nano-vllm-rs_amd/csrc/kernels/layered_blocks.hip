@@ -512,9 +512,13 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const OT *__restrict__ gu
 // divided by the sum of the chosen shares (+ 1e-20).  Rows E .. E + extra - 1 of wr are further projections of h whose values leave as they are.
 template <class OT>
 __global__ __launch_bounds__(256) void moe_route_kernel(const OT *__restrict__ h, int64_t ldh, int W, const float *__restrict__ wr, int E, int top,
-                                                        int32_t *__restrict__ sel, float *__restrict__ score, int softmax, int extra, float *__restrict__ extra_out) {
+                                                        int32_t *__restrict__ sel, float *__restrict__ score, int softmax, int extra, float *__restrict__ extra_out,
+                                                        const float *__restrict__ logits, int64_t ldl) {
     extern __shared__ float sc[];                       // [E + extra]
     const int64_t t = blockIdx.x; const int lane = threadIdx.x & 63;
+    if (logits)                                         // the products were formed by a matrix product before this launch
+        for (int e = threadIdx.x; e < E + extra; e += 256) { const float d = logits[t * ldl + e]; sc[e] = d; if (e >= E) extra_out[t * extra + (e - E)] = d; }
+    else
     for (int e = threadIdx.x >> 6; e < E + extra; e += 4) {
         float d = 0.f;
         for (int c = lane; c < W; c += 64) d = fmaf(ld_f(h, t * ldh + c), wr[(int64_t)e * W + c], d);
@@ -785,13 +789,14 @@ int silu_mul(const void *gu, int64_t T, int64_t F, void *out, int64_t ldo, bool 
 }
 
 int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr, int64_t E, int64_t top, int32_t *sel, float *score, int32_t *off, int32_t *order,
-              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s, bool softmax, int64_t extra, float *extra_out) {
+              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s, bool softmax, int64_t extra, float *extra_out,
+              const float *logits, int64_t ldl) {
     if (T == 0) return 0;
     if (extra < 0 || (extra > 0 && !extra_out)) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: %ld further rows without a place for them", (long)extra);
     if (top < 1 || top > E) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: %ld of %ld experts", (long)top, (long)E);
     if ((size_t)(E + 1) * 4 > 60000) return nvr::fail(NVR_ERR_UNSUPPORTED, "moe_route: %ld experts", (long)E);
-    if (bf16) moe_route_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), (size_t)(E + extra) * 4, s>>>((const bf16_t *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score, softmax ? 1 : 0, (int)extra, extra_out);
-    else moe_route_kernel<float><<<dim3((unsigned)T), dim3(256), (size_t)(E + extra) * 4, s>>>((const float *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score, softmax ? 1 : 0, (int)extra, extra_out);
+    if (bf16) moe_route_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), (size_t)(E + extra) * 4, s>>>((const bf16_t *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score, softmax ? 1 : 0, (int)extra, extra_out, logits, ldl);
+    else moe_route_kernel<float><<<dim3((unsigned)T), dim3(256), (size_t)(E + extra) * 4, s>>>((const float *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score, softmax ? 1 : 0, (int)extra, extra_out, logits, ldl);
     if (int rc = launched("moe_route")) return rc;
     if (pad < 1) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: rows padded to %ld", (long)pad);
     moe_group_kernel<<<dim3(1), dim3(1024), (size_t)(E + 1) * 4, s>>>(sel, (int)(T * top), (int)E, (int)pad, (int)nblocks, off, order, place_of, row_w);

@@ -94,12 +94,12 @@ __global__ __launch_bounds__(256) void conv_gates_kernel(ConvGateArgs a, Batch b
         if (st + r < 0) return 0.f;
         return hp[(int64_t)(back + r) * C + c];
     };
-    for (int c = threadIdx.x; c < C; c += 256) {
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += 256 * gridDim.y) {
         float acc = a.bias ? a.bias[c] : 0.f;
         for (int j = 0; j < taps; ++j) acc += a.w[(int64_t)c * taps + j] * input(i - back + j, c);
         st_f((OT *)a.out, (int64_t)t * a.ldo + c, silu_f(acc));
     }
-    if (threadIdx.x < a.H) {
+    if (blockIdx.y == 0 && threadIdx.x < a.H) {
         const int h = threadIdx.x;
         const float dt = softplus_f(ld_f(pr, a.dcol + h) + a.dt_bias[h]);
         a.tok_gate[((int64_t)t * a.H + h) * 2] = expf(-expf(a.a_log[h]) * dt);
@@ -107,7 +107,85 @@ __global__ __launch_bounds__(256) void conv_gates_kernel(ConvGateArgs a, Batch b
     }
     if (i == n - 1 && back > 0) {
         float *hn = a.hist + ((int64_t)(b.par[sq] ^ 1) * a.slots + b.slot[sq]) * back * C;
-        for (int idx = threadIdx.x; idx < back * C; idx += 256) { const int j = idx / C, c = idx - j * C; hn[idx] = input(n - back + j, c); }
+        for (int idx = blockIdx.y * 256 + threadIdx.x; idx < back * C; idx += 256 * gridDim.y) { const int j = idx / C, c = idx - j * C; hn[idx] = input(n - back + j, c); }
+    }
+}
+
+// 16-bit rows, 8 channels per thread as 16-byte loads and stores (C, both strides and the first column multiples of 8; 16-byte aligned rows), RB consecutive rows of
+// the step per workgroup: a thread keeps its channels' weights and the taps - 1 inputs before the current row in registers, so that every input is read once.  The
+// window is filled anew at the block's first row and at a chunk's first row (from the step's rows, the slot's history, or zeros before position 0); behind a chunk's
+// last row it holds the slot's new history.
+template <int TAPS, int RB>
+__global__ __launch_bounds__(256) void conv_gates8_kernel(ConvGateArgs a, Batch b) {
+    constexpr int BACK = TAPS - 1;
+    const int r0 = blockIdx.x * RB, r1 = min(r0 + RB, b.T), C = a.C;
+    const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+    if (blockIdx.y == 0)
+        for (int idx = threadIdx.x; idx < (r1 - r0) * a.H; idx += 256) {
+            const int t = r0 + idx / a.H, h = idx % a.H;
+            const float dt = softplus_f(ld_f((const bf16_t *)a.proj + (int64_t)t * a.ld, a.dcol + h) + a.dt_bias[h]);
+            a.tok_gate[((int64_t)t * a.H + h) * 2] = expf(-expf(a.a_log[h]) * dt);
+            a.tok_gate[((int64_t)t * a.H + h) * 2 + 1] = dt;
+        }
+    if (c0 >= C) return;
+    float wr[8][TAPS], bias[8], win[BACK > 0 ? BACK : 1][8];
+#pragma unroll
+    for (int y = 0; y < 8; ++y) {
+        bias[y] = a.bias ? a.bias[c0 + y] : 0.f;
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) wr[y][j] = a.w[(int64_t)(c0 + y) * TAPS + j];
+    }
+    auto load8 = [&](const bf16_t *p, float (&v)[8]) {
+        const uint4 u = *reinterpret_cast<const uint4 *>(p);
+        const bf16_t *e = reinterpret_cast<const bf16_t *>(&u);
+#pragma unroll
+        for (int y = 0; y < 8; ++y) v[y] = ld_f(e, y);
+    };
+    for (int t = r0; t < r1; ++t) {
+        const int sq = b.row_seq[t], i = t - b.cu[sq], n = b.cu[sq + 1] - b.cu[sq], st = b.start[sq];
+        const bf16_t *pr = (const bf16_t *)a.proj + (int64_t)t * a.ld + a.ccol + c0;
+        if (BACK > 0 && (t == r0 || i == 0)) {
+            const float *hp = a.hist + ((int64_t)b.par[sq] * a.slots + b.slot[sq]) * BACK * C;
+#pragma unroll
+            for (int j = 0; j < BACK; ++j) {
+                const int r = i - BACK + j;                 // the chunk's row of this tap (negative: before the chunk)
+                if (r >= 0) load8(pr + (int64_t)(j - BACK) * a.ld, win[j]);
+                else if (st + r < 0) {
+#pragma unroll
+                    for (int y = 0; y < 8; ++y) win[j][y] = 0.f;
+                } else {
+                    const float4 lo = *reinterpret_cast<const float4 *>(hp + (int64_t)(BACK + r) * C + c0), hi = *reinterpret_cast<const float4 *>(hp + (int64_t)(BACK + r) * C + c0 + 4);
+                    win[j][0] = lo.x; win[j][1] = lo.y; win[j][2] = lo.z; win[j][3] = lo.w; win[j][4] = hi.x; win[j][5] = hi.y; win[j][6] = hi.z; win[j][7] = hi.w;
+                }
+            }
+        }
+        float cur[8];
+        load8(pr, cur);
+        uint4 o; bf16_t *oe = reinterpret_cast<bf16_t *>(&o);
+#pragma unroll
+        for (int y = 0; y < 8; ++y) {
+            float acc = bias[y];
+#pragma unroll
+            for (int j = 0; j < BACK; ++j) acc += wr[y][j] * win[j][y];
+            acc += wr[y][BACK] * cur[y];
+            st_f(oe, y, silu_f(acc));
+        }
+        *reinterpret_cast<uint4 *>((bf16_t *)a.out + (int64_t)t * a.ldo + c0) = o;
+#pragma unroll
+        for (int j = 0; j + 1 < BACK; ++j)
+#pragma unroll
+            for (int y = 0; y < 8; ++y) win[j][y] = win[j + 1][y];
+        if (BACK > 0)
+#pragma unroll
+            for (int y = 0; y < 8; ++y) win[BACK - 1][y] = cur[y];
+        if (BACK > 0 && i == n - 1) {
+            float *hn = a.hist + ((int64_t)(b.par[sq] ^ 1) * a.slots + b.slot[sq]) * BACK * C;
+#pragma unroll
+            for (int j = 0; j < BACK; ++j) {
+                *reinterpret_cast<float4 *>(hn + (int64_t)j * C + c0) = float4{win[j][0], win[j][1], win[j][2], win[j][3]};
+                *reinterpret_cast<float4 *>(hn + (int64_t)j * C + c0 + 4) = float4{win[j][4], win[j][5], win[j][6], win[j][7]};
+            }
+        }
     }
 }
 
@@ -213,8 +291,20 @@ int pair_rows(const float *x, const float *x0, int64_t T, int64_t W, void *out, 
 int conv_gates(const ConvGateArgs &a, const Batch &b, bool bf16, hipStream_t s) {
     if (b.T == 0) return 0;
     if (a.taps < 1 || a.H > 256 || a.H < 1 || a.C < 1) return nvr::fail(NVR_ERR_INVALID_ARG, "conv_gates: %d taps over %d channels, %d heads (at most 256)", a.taps, a.C, a.H);
-    if (bf16) conv_gates_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
-    else conv_gates_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(a, b);
+    if (bf16 && a.taps <= 4 && a.C % 8 == 0 && a.ld % 8 == 0 && a.ccol % 8 == 0 && a.ldo % 8 == 0 && (((uintptr_t)a.proj | (uintptr_t)a.out | (uintptr_t)a.hist) & 15) == 0) {
+        const unsigned gy = (unsigned)((a.C / 8 + 255) / 256);
+#define NVR_CG(TAPS_)                                                                                                                                \
+        do {                                                                                                                                         \
+            if (b.T >= 1024) conv_gates8_kernel<TAPS_, 16><<<dim3((unsigned)((b.T + 15) / 16), gy), dim3(256), 0, s>>>(a, b);                         \
+            else conv_gates8_kernel<TAPS_, 1><<<dim3((unsigned)b.T, gy), dim3(256), 0, s>>>(a, b);                                                   \
+        } while (0)
+        if (a.taps == 1) NVR_CG(1); else if (a.taps == 2) NVR_CG(2); else if (a.taps == 3) NVR_CG(3); else NVR_CG(4);
+#undef NVR_CG
+        return launched("conv_gates");
+    }
+    const dim3 grid((unsigned)b.T, (unsigned)std::min<int64_t>((a.C + 255) / 256, 16));
+    if (bf16) conv_gates_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(a, b);
+    else conv_gates_kernel<float><<<grid, dim3(256), 0, s>>>(a, b);
     return launched("conv_gates");
 }
 

@@ -47,12 +47,15 @@ int LayeredModel::init_joint(nvr_model_runner &r) {
             RC(own(&w.mu, (size_t)(5 * W) * 4)); RC(own(&w.w4, (size_t)(4 * tn * W * esz))); RC(own(&w.wo2, (size_t)(W * tn * esz)));
             RC(own(&w.w0, (size_t)tn * 4)); RC(own(&w.bonus, (size_t)tn * 4)); RC(own(&w.tnorm, (size_t)tn * 4));
             if (std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) == attn_groups.end()) attn_groups.push_back(L.heads / L.kv_heads);
+            // prompts and portions on the dense graph's flash kernel in its gated form (row-major value pages)
+            w.flash = bf16 && L.dim == L.vdim && nvr::kb::flash_prefill_ok((int)L.dim, (int)L.heads, (int)L.kv_heads) && hv % 8 == 0;
+            if (w.flash && std::find(flash_groups.begin(), flash_groups.end(), L.heads / L.kv_heads) == flash_groups.end()) flash_groups.push_back(L.heads / L.kv_heads);
             max_cat = std::max(max_cat, hv); max_ro = std::max(max_ro, tn); max_t4 = std::max(max_t4, 4 * tn); max_tn = std::max(max_tn, tn);
         } else return fail(NVR_ERR_UNSUPPORTED, "layer %zu: this mixer does not belong to the joint layout", i);
         RC(named(&w.mix, (size_t)(w.nmix * W * esz)));         // (freed by name with the model)
         if (L.ff_kind == LayeredSpec::FF_MOE_GLU) {
             const int64_t f = L.expert_ff, fs = L.shared_ff;
-            RC(own(&w.router2, (size_t)((L.experts + 1) * W) * 4));
+            RC(own(&w.router_op, (size_t)(pad16(L.experts + 1) * W * esz)));      // the router's rows, then the shared expert's gate, in the operand type (zero rows behind)
             RC(own(&w.egu, (size_t)(L.experts * 2 * f * W * esz))); RC(own(&w.edown, (size_t)(L.experts * W * f * esz)));
             if (fs) { RC(own(&w.sgu, (size_t)(2 * fs * W * esz))); RC(own(&w.sdown, (size_t)(W * fs * esz))); }
             max_fs = std::max(max_fs, fs); max_top = std::max(max_top, L.top); max_e2f = std::max(max_e2f, L.top * 2 * f); max_ef = std::max(max_ef, L.top * f);
@@ -61,7 +64,7 @@ int LayeredModel::init_joint(nvr_model_runner &r) {
         max_nmix = std::max(max_nmix, w.nmix);
     }
     RC(named(&embed, (size_t)(V * W * esz))); RC(named(&head, (size_t)(V * W * esz))); RC(own(&wfinal, (size_t)W * 4));
-    if (loops) { RC(own(&loop_in, (size_t)(W * 2 * W * esz))); RC(own(&pair, (size_t)(MT * 2 * W * esz))); }
+    if (loops) { RC(own(&loop_in, (size_t)(W * 2 * W * esz))); RC(own(&pair, (size_t)(MT * 2 * W * esz))); if (bf16) RC(own(&lm_part, (size_t)(MT * ((W + 255) / 256) * 2) * 4)); }
 
     // pages for every run with attention; per slot the recurrent states and the rows before a step that the shifts and the convolution read
     size_t block_bytes = 0;
@@ -104,6 +107,7 @@ int LayeredModel::init_joint(nvr_model_runner &r) {
     const int64_t rows_e = MT * std::max<int64_t>(max_top, 1), pad_rows = (max_experts + 1) * 256;     // (experts' rows padded to whole blocks of 256)
     RC(own(&e_gu, (size_t)((MT * max_e2f + pad_rows * 2 * max_f) * esz))); RC(own(&e_act, (size_t)((MT * max_ef + pad_rows * max_f) * esz)));
     RC(own(&e_y, (size_t)((rows_e + pad_rows) * W * esz))); RC(own(&e_x, (size_t)((rows_e + pad_rows) * W * esz)));
+    RC(own(&rlogits, (size_t)(MT * pad16(max_experts + 1)) * 4));
     RC(own(&moe_i, (size_t)(3 * rows_e + max_experts + 1 + rows_e / 256 + max_experts + 1024 + 8) * 4)); RC(own(&moe_score, (size_t)rows_e * 4));
     {   // the experts' inputs are the rows as they are: a scale of one per (token, choice)
         std::vector<float> one((size_t)std::max<int64_t>(rows_e, 1), 1.0f);
@@ -125,6 +129,9 @@ int LayeredModel::load_joint(nvr_model_runner &r, const std::string &name, int d
     auto mat = [&](void *dst, int64_t ld, int64_t rows, int64_t cols) { return (dst && is2(rows, cols)) ? put(r, dst, ld, rows, cols, dtype, data, true) : bad(); };
     auto fmat = [&](float *dst, int64_t rows, int64_t cols) { return (dst && is2(rows, cols)) ? put(r, dst, cols, rows, cols, dtype, data, false) : bad(); };
     auto rows_at = [&](void *base, int64_t row0, int64_t ld) { return (void *)((char *)base + (size_t)(row0 * ld * esz)); };
+    // the decay's low-rank pair in 16 bits is kept with its rank padded by zero rows / columns to whole 256-column tiles: a product with 64 columns over many rows
+    // leaves most of the chip idle, the padded one takes the 256 x 256 tiles (tanh(0) = 0 keeps the padding out of the second product)
+    auto rank_rows = [&](int64_t rank) { return (bf16 && W % 32 == 0) ? (rank + 255) / 256 * 256 : rank; };
     if (name == "embed") return mat(embed, W, V, W);
     if (name == "head") return mat(head, W, V, W);
     if (name == "final.norm") return vec(wfinal, W);
@@ -169,21 +176,22 @@ int LayeredModel::load_joint(nvr_model_runner &r, const std::string &name, int d
         if (rest == "mix.right.w1") {                       // the rank of the decay projection is the tensor's
             if (ndim != 2 || shape[1] != W || shape[0] < 1 || (w.t_rank && w.t_rank != shape[0])) return bad();
             w.t_rank = shape[0];
-            if (!w.w1) RC(own(&w.w1, (size_t)(w.t_rank * W * esz)));
-            if (w.t_rank > tlow_cap) { RC(own(&tlow, (size_t)(r.max_tokens * w.t_rank * esz))); tlow_cap = w.t_rank; }   // (a smaller one before it stays owned)
+            const int64_t rp = rank_rows(w.t_rank);
+            if (!w.w1) RC(own(&w.w1, (size_t)(rp * W * esz)));
+            if (rp > tlow_cap) { RC(own(&tlow, (size_t)(r.max_tokens * rp * esz))); tlow_cap = rp; }   // (a smaller one before it stays owned)
             return put(r, w.w1, W, w.t_rank, W, dtype, data, true);
         }
         if (rest == "mix.right.w2") {
             if (ndim != 2 || shape[0] != tn || shape[1] < 1 || (w.t_rank && w.t_rank != shape[1])) return bad();
             w.t_rank = shape[1];
-            if (!w.w2) RC(own(&w.w2, (size_t)(tn * w.t_rank * esz)));
-            return put(r, w.w2, w.t_rank, tn, w.t_rank, dtype, data, true);
+            if (!w.w2) RC(own(&w.w2, (size_t)(tn * rank_rows(w.t_rank) * esz)));
+            return put(r, w.w2, rank_rows(w.t_rank), tn, w.t_rank, dtype, data, true);
         }
     }
     if (L.ff_kind == LayeredSpec::FF_MOE_GLU) {
         const int64_t f = L.expert_ff, fs = L.shared_ff;
-        if (rest == "mlp.router") return fmat(w.router2, L.experts, W);
-        if (fs && rest == "mlp.shared.sg") return fmat(w.router2 + L.experts * W, 1, W);
+        if (rest == "mlp.router") return mat(w.router_op, W, L.experts, W);
+        if (fs && rest == "mlp.shared.sg") return mat(rows_at(w.router_op, L.experts, W), W, 1, W);
         if (fs && rest == "mlp.shared.gate") return mat(w.sgu, W, fs, W);
         if (fs && rest == "mlp.shared.up") return mat(rows_at(w.sgu, fs, W), W, fs, W);
         if (fs && rest == "mlp.shared.down") return mat(w.sdown, fs, W, fs);
@@ -214,7 +222,11 @@ int LayeredModel::forward_joint(nvr_model_runner &r, const StepPlan &p) {
         const LayeredSpec::Layer &L = spec.layers[li]; const LayerW &w = lw[li]; RunState &st = rs[(size_t)ri];
         if (spec.pass_start[(size_t)ri]) {                   // a pass over the looped range starts from the stream and the embedding output together
             RC(kl::pair_rows(x, x0, T, W, pair, bf16, s));
-            RC(gemm(r, pair, 2 * W, loop_in, T, 2 * W, W, x, true));
+            if (bf16 && lm_part && nvr::kb::gemm256_lm_head_ok(T, 2 * W, W, 2 * W)) {       // many rows: the 256 x 256 product that leaves in f32 (the LM head's; its arg-max partials are not read)
+                int32_t nparts = 0;
+                RC(nvr::kb::gemm256_lm_head((const uint16_t *)pair, 2 * W, (const uint16_t *)loop_in, T, 2 * W, W, x, lm_part, (int32_t *)(lm_part + MT * ((W + 255) / 256)), &nparts, s));
+            } else
+                RC(gemm(r, pair, 2 * W, loop_in, T, 2 * W, W, x, true));
         }
         RC(kl::norm_shift(x, b, W, eps, w.n1, w.shift, L.has_mlp ? a2 : nullptr, a1, st.hist, slots, bf16, s));
         RC(gemm(r, a1, W, w.mix, T, W, w.nmix, proj));
@@ -240,12 +252,21 @@ int LayeredModel::forward_joint(nvr_model_runner &r, const StepPlan &p) {
             kl::SinkAttnArgs a{};
             a.q = at(proj, w.qcol); a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.chunk = (int32_t)L.chunk; a.softcap = (float)L.softcap; a.gate_bias = w.pb;
             a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale; a.out = cat; a.ldo = hv;
-            a.v_grouped = 1;
+            a.v_grouped = w.flash ? 0 : 1;                                           // (a property of the layer: the pages keep one layout)
             const bool tiled = kl::sink_attention_tiled_ok(a, bf16, (int)r.block_size);       // (a property of the layer's shape: the pages keep one layout)
             kl::RopeStoreArgs ra{}; ra.proj = proj; ra.ld = w.nmix; ra.qcol = w.qcol; ra.kcol = w.kcol; ra.vcol = w.vcol; ra.H = a.H; ra.G = a.G; ra.D = a.D; ra.Dv = a.Dv;
-            ra.rot = (int32_t)L.rot_dims; ra.freq = w.rfreq; ra.kc = st.kc; ra.vc = st.vc; ra.v_grouped = tiled;
+            ra.rot = (int32_t)L.rot_dims; ra.freq = w.rfreq; ra.kc = st.kc; ra.vc = st.vc; ra.v_grouped = tiled && !w.flash;
             RC(kl::rope_store(ra, b, bf16, s));
-            if (tiled) {
+            if (w.flash && !p.decode_sized) {
+                const size_t gi = (size_t)(std::find(flash_groups.begin(), flash_groups.end(), L.heads / L.kv_heads) - flash_groups.begin());
+                nvr::kt::FlashArgs f{};
+                f.q = (const uint16_t *)a.q; f.ldq = w.nmix; f.k = (const uint16_t *)st.kc; f.v = (const uint16_t *)st.vc; f.ldkv = 0;
+                f.block_tables = b.block_tables; f.max_blocks = b.max_blocks; f.block_size = b.block_size;
+                f.tiles = (const nvr::kt::FlashTile *)(in_dev + p.o_ftiles[gi]); f.ntiles = p.n_ftiles[gi];
+                f.H = (int32_t)L.heads; f.KVH = (int32_t)L.kv_heads; f.D = (int32_t)L.dim; f.scale = (float)L.scale; f.out = (uint16_t *)cat; f.ldo = hv;
+                f.gate_bias = w.pb; f.softcap = (float)L.softcap; f.chunk = (int32_t)L.chunk;
+                RC(nvr::kb::flash_prefill(f, true, s));
+            } else if (tiled) {
                 const size_t gi = (size_t)(std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) - attn_groups.begin());
                 // decode-sized steps over long chunks: few tiles, many keys each — a tile's keys go to several workgroups whose partial sums are added up
                 const int64_t wgs = (int64_t)p.n_tiles[gi] * L.kv_heads, keys = L.chunk > 0 ? std::min<int64_t>(p.max_ctx, L.chunk + 64) : p.max_ctx;
@@ -258,17 +279,24 @@ int LayeredModel::forward_joint(nvr_model_runner &r, const StepPlan &p) {
             RC(gemm(r, cat, hv, w.wo, T, hv, W, tmp));
             // right: five shifted inputs, their projections (one matrix per input), the decay's two products, retention's gated form with a bonus
             RC(kl::shift_mixes(a1, W, b, W, 5, w.mu, mixes, st.shist, slots, bf16, s));
-            kl::HeadLinearArgs ha{}; ha.a = mixes; ha.lda = 5 * W; ha.ha = W; ha.w = w.w4; ha.y = tproj; ha.ldy = 4 * tn; ha.hy = tn; ha.T = (int32_t)T; ha.H = 4; ha.K = (int32_t)W; ha.N = (int32_t)tn;
-            RC(kl::head_linear(ha, bf16, s));
-            RC(gemm(r, at(mixes, 4 * W), 5 * W, w.w1, T, W, w.t_rank, tlow));
-            RC(kl::tanh_rows(tlow, w.t_rank, T, w.t_rank, bf16, s));
-            RC(gemm(r, tlow, w.t_rank, w.w2, T, w.t_rank, tn, tz));
+            // r, k, v, g leave in planes of [max tokens][Ht Dt] each: many rows take the tiled product once per plane, few rows one launch with a matrix per plane
+            const int64_t plane = MT * tn;
+            if (T >= 128) {
+                for (int k = 0; k < 4; ++k) RC(gemm(r, at(mixes, k * W), 5 * W, at(w.w4, k * tn * W), T, W, tn, at(tproj, k * plane)));
+            } else {
+                kl::HeadLinearArgs ha{}; ha.a = mixes; ha.lda = 5 * W; ha.ha = W; ha.w = w.w4; ha.y = tproj; ha.ldy = tn; ha.hy = plane; ha.T = (int32_t)T; ha.H = 4; ha.K = (int32_t)W; ha.N = (int32_t)tn;
+                RC(kl::head_linear(ha, bf16, s));
+            }
+            const int64_t rp = (bf16 && W % 32 == 0) ? (w.t_rank + 255) / 256 * 256 : w.t_rank;       // (the rank as load_joint padded it)
+            RC(gemm(r, at(mixes, 4 * W), 5 * W, w.w1, T, W, rp, tlow));
+            RC(kl::tanh_rows(tlow, rp, T, rp, bf16, s));
+            RC(gemm(r, tlow, rp, w.w2, T, rp, tn, tz));
             kl::RetentionArgs t{};
-            t.proj = tproj; t.ld = 4 * tn; t.qcol = 0; t.kcol = tn; t.vcol = 2 * tn; t.rot_dims = 0; t.kscale = 1.0f; t.qscale = 1.0f; t.inv_tau = 1.f;
+            t.proj = tproj; t.ld = tn; t.qcol = 0; t.kcol = plane; t.vcol = 2 * plane; t.rot_dims = 0; t.kscale = 1.0f; t.qscale = 1.0f; t.inv_tau = 1.f;
             t.H = (int32_t)L.t_heads; t.D = (int32_t)L.t_dim; t.Dv = (int32_t)L.t_dim; t.az = tz; t.ldz = tn; t.abias = w.w0; t.decay_exp = true; t.bonus = w.bonus;
             t.state = st.state; t.o = ret_o;
             RC(kl::retention(t, b, bf16, s));
-            RC(kl::head_norm_gate(ret_o, tproj, 4 * tn, 3 * tn, T, L.t_heads, L.t_dim, eps, w.tnorm, tcat, tn, bf16, s, true));
+            RC(kl::head_norm_gate(ret_o, tproj, tn, 3 * plane, T, L.t_heads, L.t_dim, eps, w.tnorm, tcat, tn, bf16, s, true));
             RC(gemm(r, tcat, tn, w.wo2, T, tn, W, tmp2));
             j.w1 = w.outl; j.y2 = tmp2; j.ld2 = W; j.w2 = w.outr;
         }
@@ -278,8 +306,11 @@ int LayeredModel::forward_joint(nvr_model_runner &r, const StepPlan &p) {
             // many rows: every expert's rows padded to whole blocks of 256, brought together once, and the dense graph's 256 x 256 product with a matrix per row block
             const int64_t nblocks = n / 256 + L.experts;
             const bool blocks = bf16 && n >= 2048 && nvr::kb::gemm256_ok(nblocks * 256, W, 2 * f, W) && nvr::kb::gemm256_ok(nblocks * 256, f, W, f);
-            RC(kl::moe_route(a2, W, T, W, w.router2, L.experts, L.top, sel, moe_score, off, order, place_of, blocks ? 256 : 1, blocks ? row_w : nullptr, nblocks, bf16, s,
-                             true, fs ? 1 : 0, fs ? shared_g : nullptr));
+            // router logits (and the shared expert's gate): one product with f32 accumulation that leaves in f32, then the choice per token
+            const int64_t ne = pad16(L.experts + 1);
+            RC(gemm(r, a2, W, w.router_op, T, W, ne, rlogits, true));
+            RC(kl::moe_route(a2, W, T, W, nullptr, L.experts, L.top, sel, moe_score, off, order, place_of, blocks ? 256 : 1, blocks ? row_w : nullptr, nblocks, bf16, s,
+                             true, fs ? 1 : 0, fs ? shared_g : nullptr, rlogits, ne));
             if (blocks) {
                 RC(kl::moe_gather(a2, W, T, W, L.top, place_of, gfloor, e_x, bf16, s));
                 RC(nvr::kb::gemm256_grouped((const uint16_t *)e_x, W, (const uint16_t *)w.egu, 2 * f * W, row_w, nblocks * 256, W, 2 * f, (uint16_t *)e_gu, s));

@@ -126,7 +126,7 @@ public:
         float *pb = nullptr; float *mu = nullptr;                                    // attention's bias per head; the five mixes' blends [5][W]
         void *w4 = nullptr, *w1 = nullptr, *w2 = nullptr; int64_t t_rank = 0;         // time mixing: r / k / v / g stacked [4][Ht Dt][W]; decay projections [rank][W], [Ht Dt][rank]
         float *w0 = nullptr, *bonus = nullptr, *tnorm = nullptr;                      // [Ht Dt] each
-        float *router2 = nullptr;                                                    // [E + 1][W] f32: the router's rows, then the shared expert's gate
+        void *router_op = nullptr;                                                   // [E + 1, padded to 16][W] operand type: the router's rows, then the shared expert's gate
     };
     struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; void *rows = nullptr; float *mstate = nullptr;
                       float *shist = nullptr, *chist = nullptr; };   // joint layout: hist the norm output before the step [2][slots][W], shist the mixer input's (time mixing), chist the convolution's inputs   // mstate: a matrix memory's running maxima [slots][H]   // borrowed: another run's pages (a shared latent)
@@ -146,7 +146,8 @@ public:
     // joint layout
     void *loop_in = nullptr, *pair = nullptr; float *x0 = nullptr;          // [W][2 W]; [max tokens][2 W] operand rows; the embedding output
     void *conv_o = nullptr, *mixes = nullptr, *tproj = nullptr, *tlow = nullptr, *tz = nullptr, *tcat = nullptr; float *shared_g = nullptr;
-    int64_t tlow_cap = 0;
+    int64_t tlow_cap = 0; float *rlogits = nullptr;                          // router logits of a step [max tokens][experts + 1, padded]
+    float *lm_part = nullptr;                          // arg-max partials of the 256 x 256 product with f32 output (not read)
     std::vector<void *> owned;                                              // device allocations of the sequential layout (freed with the model)
     // activations
     float *x = nullptr, *ret_o = nullptr;                                  // residual stream, retention outputs: f32

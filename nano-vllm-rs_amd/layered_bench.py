@@ -1,4 +1,4 @@
-"""Prefill and decode throughput of the layer-list designs (Rugudra, Pusunex, Sosutar) beside the dense Qwen3 graph at equal sizes (bench.py --layered-compare).
+"""Prefill and decode throughput of the layer-list designs (Rugudra, Pusunex, Sosutar, Sokalorn) beside the dense Qwen3 graph at equal sizes (bench.py --layered-compare).
 
 Random weights, layer shapes that resemble a real model's; both models go through the same engine (scheduler, block manager, runner step).
 Per size one JSON object: tokens/s of one prefill step over BATCH prompts of PROMPT tokens and of the decode steps that follow, for both."""
@@ -175,6 +175,59 @@ def sosutar_weights(cfg, seed=0):
     return out
 
 
+def sokalorn_config(s, chunk=512):
+    """A state-space layer and an attention over chunks beside a time mixing, both with eight experts of ff / 4 (two per token) and a shared expert of ff / 2; the pair
+    runs layers / 2 times with the same weights, every pass behind the product over [x ; embedding output]."""
+    H, G, D, W = s["heads"], s["kv_heads"], s["dim"], s["width"]
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"] // 4, "limit": 7.0}, "router": {"experts": 8, "top": 2}, "shared": {"ff": s["ff"] // 2, "limit": 7.0}}
+    layers = [{"type": "mamba2", "mixer": {"heads": H, "vdim": D, "state": 128, "groups": G, "conv": 4, "norm_groups": G}, "mlp": mlp},
+              {"type": "parallel", "mixer": {"left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "mask": {"size": chunk}, "scale": D ** -0.5, "softcap": 30.0,
+                                                      "rot": {"dims": D // 2, "base": 10000.0, "scaling": {"factor": 4.0}}},
+                                             "right": {"heads": W // 64, "dim": 64}}, "mlp": mlp}]
+    return {"architecture": "Sokalorn", "vocab": s["vocab"], "width": W, "norm": {"eps": 1e-5}, "layers": layers, "loop": {"start": 0, "stop": 2, "times": max(1, s["layers"] // 2)}}
+
+
+def sokalorn_weights(cfg, seed=0, t_rank=64):
+    rng = np.random.default_rng(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def lin(o, i, g=1.0):
+        return (rng.standard_normal((o, i), dtype=np.float32) * (g / np.sqrt(i))).astype(np.float32)
+
+    def gains(n, mean=1.0):
+        return (mean + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    out = {"embed": rng.standard_normal((V, W), dtype=np.float32), "head": lin(V, W), "final.norm": gains(W), "loop.in": lin(W, 2 * W)}
+    for i, L in enumerate(cfg["layers"]):
+        m, p = L["mixer"], "l%d." % i
+        out[p + "norm1"], out[p + "shift"] = gains(W), rng.uniform(0.0, 1.0, W).astype(np.float32)
+        if L["type"] == "mamba2":
+            H, P, N, G, taps = m["heads"], m["vdim"], m["state"], m["groups"], m["conv"]
+            C = H * P + 2 * G * N
+            out[p + "mix.in"], out[p + "mix.conv"], out[p + "mix.conv.b"] = lin(2 * H * P + 2 * G * N + H, W), (0.5 * rng.standard_normal((C, taps))).astype(np.float32), (0.1 * rng.standard_normal(C)).astype(np.float32)
+            out[p + "mix.dt_bias"], out[p + "mix.A_log"] = rng.uniform(-4.0, -1.0, H).astype(np.float32), rng.uniform(-1.0, 1.0, H).astype(np.float32)
+            out[p + "mix.D"], out[p + "mix.norm"], out[p + "mix.o"] = rng.standard_normal(H).astype(np.float32), gains(H * P), lin(W, H * P)
+        else:
+            a, t = m["left"], m["right"]
+            H, G, D, Dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            q = p + "mix.left."
+            out[q + "q"], out[q + "k"], out[q + "v"], out[q + "g"], out[q + "o"] = lin(H * D, W), lin(G * D, W), lin(G * Dv, W), lin(H * Dv, W), lin(W, H * Dv)
+            out[q + "pb"], out[q + "out"] = rng.uniform(-6.0, -3.0, H).astype(np.float32), gains(W)
+            q, tn = p + "mix.right.", t["heads"] * t["dim"]
+            for c in "rkvgw":
+                out[q + "mu." + c] = rng.uniform(0.0, 1.0, W).astype(np.float32)
+            out[q + "r"], out[q + "k"], out[q + "v"], out[q + "g"], out[q + "o"] = lin(tn, W), lin(tn, W), lin(tn, W), lin(tn, W), lin(W, tn)
+            out[q + "w1"], out[q + "w2"], out[q + "w0"] = lin(t_rank, W), lin(tn, t_rank), rng.uniform(-5.0, -1.0, tn).astype(np.float32)
+            out[q + "u"], out[q + "norm"], out[q + "out"] = (0.5 * rng.standard_normal((t["heads"], t["dim"]))).astype(np.float32), gains(tn), gains(W)
+        mlp = L.get("mlp")
+        if mlp:
+            E = mlp["router"]["experts"]
+            out[p + "mlp.router"], out[p + "mlp.shared.sg"] = lin(E, W), lin(1, W)
+            for n in ["e%d" % e for e in range(E)] + ["shared"]:
+                f = mlp["shared"]["ff"] if n == "shared" else mlp["expert"]["ff"]
+                out[p + "mlp.%s.gate" % n], out[p + "mlp.%s.up" % n], out[p + "mlp.%s.down" % n] = lin(f, W), lin(f, W), lin(W, f)
+    return out
+
+
 def _run(nvr, engine, vocab, batch, prompt, steps, warmup):
     sp = nvr.SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True)
     for i in range(batch):
@@ -228,6 +281,14 @@ def compare(nvr, sizes=("w1024", "w2048"), batch=16, prompt=1024, steps=32, warm
                 eng.model_runner.load_tensor(k, np.asarray(v))
             _run(nvr, eng, s["vocab"], 2, 64, 2, 1)
             line["sosutar"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
+            del eng
+        if "sokalorn" in which:
+            cfg = sokalorn_config(s)
+            eng = nvr.LLMEngine(nvr.Config(**ecfg), nvr.ModelSpec(cfg))
+            for k, v in sokalorn_weights(cfg).items():
+                eng.model_runner.load_tensor(k, np.asarray(v))
+            _run(nvr, eng, s["vocab"], 2, 64, 2, 1)
+            line["sokalorn"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
             del eng
         if "qwen3" in which:
             m = nvr.ModelConfig(vocab_size=s["vocab"], hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
