@@ -263,6 +263,42 @@ __global__ __launch_bounds__(256) void shift_mixes_kernel(const OT *__restrict__
     }
 }
 
+// 16-bit rows, 8 channels per thread as 16-byte loads and stores (W and the stride multiples of 8, 16-byte aligned rows)
+__global__ __launch_bounds__(256) void shift_mixes8_kernel(const bf16_t *__restrict__ m, int64_t ldm, Batch b, int W, int nm, const float *__restrict__ mu, bf16_t *__restrict__ out,
+                                                           float *__restrict__ hist, int64_t slots) {
+    const int t = blockIdx.x, sq = b.row_seq[t];
+    const int i = t - b.cu[sq], n = b.cu[sq + 1] - b.cu[sq], st = b.start[sq];
+    const bf16_t *mr = m + (int64_t)t * ldm;
+    const float *hp = (i == 0 && st > 0) ? hist + ((int64_t)b.par[sq] * slots + b.slot[sq]) * W : nullptr;
+    float *hn = i == n - 1 ? hist + ((int64_t)(b.par[sq] ^ 1) * slots + b.slot[sq]) * W : nullptr;
+    bf16_t *orow = out + (int64_t)t * nm * W;
+    for (int c0 = threadIdx.x * 8; c0 < W; c0 += 256 * 8) {
+        float v[8], before[8];
+        const uint4 u = *reinterpret_cast<const uint4 *>(mr + c0);
+        const bf16_t *e = reinterpret_cast<const bf16_t *>(&u);
+#pragma unroll
+        for (int y = 0; y < 8; ++y) v[y] = ld_f(e, y);
+        if (i > 0) {
+            const uint4 p = *reinterpret_cast<const uint4 *>(mr - ldm + c0);
+            const bf16_t *pe = reinterpret_cast<const bf16_t *>(&p);
+#pragma unroll
+            for (int y = 0; y < 8; ++y) before[y] = ld_f(pe, y);
+        } else {
+#pragma unroll
+            for (int y = 0; y < 8; ++y) before[y] = hp ? hp[c0 + y] : 0.f;
+        }
+        for (int k = 0; k < nm; ++k) {
+            uint4 o; bf16_t *oe = reinterpret_cast<bf16_t *>(&o);
+#pragma unroll
+            for (int y = 0; y < 8; ++y) st_f(oe, y, v[y] + (before[y] - v[y]) * mu[(int64_t)k * W + c0 + y]);
+            *reinterpret_cast<uint4 *>(orow + (int64_t)k * W + c0) = o;
+        }
+        if (hn)
+#pragma unroll
+            for (int y = 0; y < 8; ++y) hn[c0 + y] = v[y];
+    }
+}
+
 template <class OT>
 __global__ __launch_bounds__(256) void tanh_rows_kernel(OT *__restrict__ y, int64_t ld, int64_t T, int64_t N) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -327,7 +363,9 @@ int rope_store(const RopeStoreArgs &a, const Batch &b, bool bf16, hipStream_t s)
 
 int shift_mixes(const void *m, int64_t ldm, const Batch &b, int64_t W, int32_t n, const float *mu, void *out, float *hist, int64_t slots, bool bf16, hipStream_t s) {
     if (b.T == 0) return 0;
-    if (bf16) shift_mixes_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)m, ldm, b, (int)W, (int)n, mu, (bf16_t *)out, hist, slots);
+    if (bf16 && W % 8 == 0 && ldm % 8 == 0 && (((uintptr_t)m | (uintptr_t)out) & 15) == 0)
+        shift_mixes8_kernel<<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)m, ldm, b, (int)W, (int)n, mu, (bf16_t *)out, hist, slots);
+    else if (bf16) shift_mixes_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)m, ldm, b, (int)W, (int)n, mu, (bf16_t *)out, hist, slots);
     else shift_mixes_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const float *)m, ldm, b, (int)W, (int)n, mu, (float *)out, hist, slots);
     return launched("shift_mixes");
 }
