@@ -266,13 +266,16 @@ __global__ __launch_bounds__(256) void shift_mixes_kernel(const OT *__restrict__
 // 16-bit rows, 8 channels per thread as 16-byte loads and stores (W and the stride multiples of 8, 16-byte aligned rows)
 __global__ __launch_bounds__(256) void shift_mixes8_kernel(const bf16_t *__restrict__ m, int64_t ldm, Batch b, int W, int nm, const float *__restrict__ mu, bf16_t *__restrict__ out,
                                                            float *__restrict__ hist, int64_t slots) {
-    const int t = blockIdx.x, sq = b.row_seq[t];
+    const int w8 = W >> 3;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;       // (row, piece of 8 channels): every thread has its own piece
+    if (idx >= (int64_t)b.T * w8) return;
+    const int t = (int)(idx / w8), c0 = (int)(idx - (int64_t)t * w8) << 3, sq = b.row_seq[t];
     const int i = t - b.cu[sq], n = b.cu[sq + 1] - b.cu[sq], st = b.start[sq];
     const bf16_t *mr = m + (int64_t)t * ldm;
     const float *hp = (i == 0 && st > 0) ? hist + ((int64_t)b.par[sq] * slots + b.slot[sq]) * W : nullptr;
     float *hn = i == n - 1 ? hist + ((int64_t)(b.par[sq] ^ 1) * slots + b.slot[sq]) * W : nullptr;
     bf16_t *orow = out + (int64_t)t * nm * W;
-    for (int c0 = threadIdx.x * 8; c0 < W; c0 += 256 * 8) {
+    {
         float v[8], before[8];
         const uint4 u = *reinterpret_cast<const uint4 *>(mr + c0);
         const bf16_t *e = reinterpret_cast<const bf16_t *>(&u);
@@ -285,17 +288,24 @@ __global__ __launch_bounds__(256) void shift_mixes8_kernel(const bf16_t *__restr
             for (int y = 0; y < 8; ++y) before[y] = ld_f(pe, y);
         } else {
 #pragma unroll
-            for (int y = 0; y < 8; ++y) before[y] = hp ? hp[c0 + y] : 0.f;
+            for (int y = 0; y < 8; ++y) before[y] = 0.f;
+            if (hp) {
+                const float4 h0 = *reinterpret_cast<const float4 *>(hp + c0), h1 = *reinterpret_cast<const float4 *>(hp + c0 + 4);
+                before[0] = h0.x; before[1] = h0.y; before[2] = h0.z; before[3] = h0.w; before[4] = h1.x; before[5] = h1.y; before[6] = h1.z; before[7] = h1.w;
+            }
         }
         for (int k = 0; k < nm; ++k) {
             uint4 o; bf16_t *oe = reinterpret_cast<bf16_t *>(&o);
+            const float4 m0 = *reinterpret_cast<const float4 *>(mu + (int64_t)k * W + c0), m1 = *reinterpret_cast<const float4 *>(mu + (int64_t)k * W + c0 + 4);
+            const float mk[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
 #pragma unroll
-            for (int y = 0; y < 8; ++y) st_f(oe, y, v[y] + (before[y] - v[y]) * mu[(int64_t)k * W + c0 + y]);
+            for (int y = 0; y < 8; ++y) st_f(oe, y, v[y] + (before[y] - v[y]) * mk[y]);
             *reinterpret_cast<uint4 *>(orow + (int64_t)k * W + c0) = o;
         }
-        if (hn)
-#pragma unroll
-            for (int y = 0; y < 8; ++y) hn[c0 + y] = v[y];
+        if (hn) {
+            *reinterpret_cast<float4 *>(hn + c0) = float4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<float4 *>(hn + c0 + 4) = float4{v[4], v[5], v[6], v[7]};
+        }
     }
 }
 
@@ -363,8 +373,8 @@ int rope_store(const RopeStoreArgs &a, const Batch &b, bool bf16, hipStream_t s)
 
 int shift_mixes(const void *m, int64_t ldm, const Batch &b, int64_t W, int32_t n, const float *mu, void *out, float *hist, int64_t slots, bool bf16, hipStream_t s) {
     if (b.T == 0) return 0;
-    if (bf16 && W % 8 == 0 && ldm % 8 == 0 && (((uintptr_t)m | (uintptr_t)out) & 15) == 0)
-        shift_mixes8_kernel<<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)m, ldm, b, (int)W, (int)n, mu, (bf16_t *)out, hist, slots);
+    if (bf16 && W % 8 == 0 && ldm % 8 == 0 && (((uintptr_t)m | (uintptr_t)out | (uintptr_t)mu | (uintptr_t)hist) & 15) == 0)
+        shift_mixes8_kernel<<<dim3((unsigned)(((int64_t)b.T * (W / 8) + 255) / 256)), dim3(256), 0, s>>>((const bf16_t *)m, ldm, b, (int)W, (int)n, mu, (bf16_t *)out, hist, slots);
     else if (bf16) shift_mixes_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)m, ldm, b, (int)W, (int)n, mu, (bf16_t *)out, hist, slots);
     else shift_mixes_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const float *)m, ldm, b, (int)W, (int)n, mu, (float *)out, hist, slots);
     return launched("shift_mixes");

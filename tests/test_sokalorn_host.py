@@ -106,7 +106,7 @@ def test_the_bonus_reaches_the_current_token_only():
 
 
 def test_the_probe_key_decides_its_row_inside_the_chunk_only():
-    cfg = make_config([side_layer(heads=4, kv_heads=2, dim=16, vdim=16, chunk=20, scale=0.25, softcap=20.0, t_heads=1, t_dim=8, mlp=None)], vocab=31, width=48)
+    cfg = make_config([side_layer(heads=4, kv_heads=2, dim=16, vdim=16, chunk=20, scale=0.25, softcap=24.0, t_heads=1, t_dim=8, mlp=None)], vocab=31, width=48)
     Q, K = 0, 1
     w = make_key_stand_out(cfg, make_weights(cfg, seed=4), Q, K)
     w["l0.mix.right.out"] = np.zeros_like(w["l0.mix.right.out"]); w["l0.mix.right.mu.r"] = np.zeros_like(w["l0.mix.right.mu.r"])
