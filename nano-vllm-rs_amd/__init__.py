@@ -357,7 +357,7 @@ class ModelConfig:
 
 class ModelSpec:
     """A checkpoint's config.json as the model registry reads it (nvr_model_spec_from_json): which family runs the architecture it names —
-    0 the dense Qwen3 graph (ModelConfig), 1 a list of layers (Rugudra, Pusunex, Sosutar) — and that family's description.  `ModelSpec.from_pretrained(dir)` reads
+    0 the dense Qwen3 graph (ModelConfig), 1 a list of layers (Rugudra, Pusunex, Sosutar, Sokalorn) — and that family's description.  `ModelSpec.from_pretrained(dir)` reads
     dir/config.json; `ModelSpec(dict_or_text)` takes the configuration itself."""
 
     def __init__(self, config):

@@ -53,7 +53,7 @@ def test_every_cited_abi_symbol_and_test_name_exists():
         for name, is_prefix in _cited(text, "test_"):
             if name in ("test_", "test_tp", "test_kernels_gpu", "test_engine_gpu", "test_host_parity", "test_oracle_kat", "test_golden", "test_scale", "test_weights",
                         "test_tokenizer", "test_ctrl", "test_bf16_gpu", "test_kernels_bf16_gpu", "test_kernels_f32_gpu", "test_baseline_parity", "test_sanitizers",
-                        "test_bench_counters", "test_design_refs", "test_rugudra_host", "test_rugudra_gpu", "test_pusunex_host", "test_pusunex_gpu", "test_sosutar_host", "test_sosutar_gpu"):
+                        "test_bench_counters", "test_design_refs", "test_rugudra_host", "test_rugudra_gpu", "test_pusunex_host", "test_pusunex_gpu", "test_sosutar_host", "test_sosutar_gpu", "test_sokalorn_host", "test_sokalorn_gpu"):
                 continue                                                  # file names
             ok = any(t.startswith(name) for t in tests) if is_prefix else name in tests
             if not ok and any(t.startswith(name) for t in tests) and len(name) >= 24:
